@@ -649,9 +649,18 @@ struct Access {
     std::string view;   // type, shape, strides, offsets, padded shape: equal views address alike
     ark::Dims shape;
     int step = -1;      // schedule step of the task group that makes the access
+    // True when task t of the op touches only tile t of this tensor: every access of a
+    // tiled elementwise op, and the *result* of a matmul.  A matmul task reads a whole
+    // row panel of its first operand and a column panel of its second, whoever wrote them.
+    bool tile_local = false;
+    // A read that spans more than the reading task's own part of the tensor (the
+    // operands of a matmul or of attention): never a workgroup-local matter.
+    bool panel_read = false;
 };
 
-void add_access(std::vector<Access> &out, const Json &tensor_json, bool write) {
+bool tiled_elementwise(const std::string &type);
+
+void add_access(std::vector<Access> &out, const Json &tensor_json, bool write, const std::string &op_type) {
     auto t = ark::ModelTensor::deserialize(tensor_json);
     ark::Dims st = t->strides(), pd = t->padded_shape();
     size_t last = 0, pitch = 1;
@@ -661,6 +670,8 @@ void add_access(std::vector<Access> &out, const Json &tensor_json, bool write) {
     }
     const size_t elem = t->data_type()->bytes();
     Access a{t->buffer()->id(), t->byte_offset(), t->byte_offset() + (last + 1) * elem, write, "", t->shape(), -1};
+    a.tile_local = tiled_elementwise(op_type) || (write && op_type == "Matmul");
+    a.panel_read = !write && (op_type == "Matmul" || op_type == "MatmulSwiglu" || op_type == "Attention");
     a.view = tensor_json.at("DataType").dump() + tensor_json.at("Shape").dump() + tensor_json.at("Strides").dump() +
              tensor_json.at("Offsets").dump() + tensor_json.at("PaddedShape").dump();
     out.push_back(a);
@@ -669,9 +680,10 @@ void add_access(std::vector<Access> &out, const Json &tensor_json, bool write) {
 std::vector<Access> accesses_of(const Json &task_info) {
     std::vector<Access> v;
     for (const auto &op : task_info.at("Ops").elements()) {
-        for (const auto &t : op.at("ReadTensors").elements()) add_access(v, t, false);
-        for (const auto &t : op.at("WriteTensors").elements()) add_access(v, t, true);
-        for (const auto &t : op.at("ResultTensors").elements()) add_access(v, t, true);
+        const std::string type = op.at("Type").as_string();
+        for (const auto &t : op.at("ReadTensors").elements()) add_access(v, t, false, type);
+        for (const auto &t : op.at("WriteTensors").elements()) add_access(v, t, true, type);
+        for (const auto &t : op.at("ResultTensors").elements()) add_access(v, t, true, type);
     }
     return v;
 }
@@ -909,12 +921,15 @@ struct Executor {
             for (auto &x : a) x.step = (int)sj;
             return a;
         };
-        // A dependency is local to a workgroup when producer and consumer are
-        // elementwise ops with the same tiling and the shared tensor is seen
-        // through the same view and has the output's shape in both: the elements
-        // task t reads are the ones task t of the other op wrote, on the same
-        // workgroup.  Such a dependency needs no grid barrier.
+        // A dependency is local to a workgroup when both ops cut equal output shapes
+        // into the same tiles on the same workgroups, both touch the shared tensor
+        // tile by tile (an elementwise op, or a matmul as the writer: never a matmul's
+        // operand reads, which span whole panels), and both see it through the same
+        // view with the output's shape: the elements task t reads are the ones task t
+        // of the other op wrote, on the same workgroup.  Such a dependency needs no
+        // grid barrier.
         auto local_pair = [&](const Access &x, const Access &y) {
+            if (!x.tile_local || !y.tile_local) return false;
             const auto &sx = sched.steps[(size_t)x.step];
             const auto &sy = sched.steps[(size_t)y.step];
             const Json &tx = task_infos.at((size_t)sx.task_info), &ty = task_infos.at((size_t)sy.task_info);
@@ -1071,7 +1086,7 @@ struct Executor {
                         if (has_scratch(x.step) || has_scratch(y.step))
                             local = false;
                         else if (x.step == y.step)
-                            local = x.view == y.view && x.begin == y.begin;
+                            local = !x.panel_read && !y.panel_read && x.view == y.view && x.begin == y.begin;
                         else
                             local = local_pair(x, y);
                         if (!local) all_local = false;
@@ -1315,6 +1330,9 @@ struct Executor {
             es[i] = acc;
             acc *= st[i];
         }
+        for (int i = 0; i < 4; ++i)
+            if (sh[i] < 0 || of[i] < 0 || st[i] < 1 || of[i] + sh[i] > st[i])
+                ARK_ERR(InvalidUsageError, "tensor view: offset + shape exceeds the stride in dimension ", i - (4 - ndims));
         if ((size_t)acc * elem > buffer_bytes.at(buffer_id))
             ARK_ERR(InvalidUsageError, "tensor view exceeds its buffer");
         char *base = arena + it->second +

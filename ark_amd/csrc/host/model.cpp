@@ -212,82 +212,98 @@ void Model::noop(Tensor input, const std::string &name) {
     impl_->add_named_op(op, name);
 }
 
-// Stride/offset inference of a reshaped view (ark/ops/ops_reshape.cpp:16-132):
-// walk both shapes from the innermost dimension, merging or splitting
-// dimensions; a dimension of the input may only be merged into a larger one
-// when it is dense (stride == shape, offset 0).
+// Stride/offset inference of a reshaped view (results as ark/ops/ops_reshape.cpp:16-132).
+//
+// The rule: read innermost-first, the old and the new shape fall into runs of
+// dimensions with equal element counts (a run closes as soon as the two counts
+// agree).  Inside a run
+//   * every old dimension but the outermost must be dense (stride == extent,
+//     offset 0): only then do the run's old dimensions address one contiguous
+//     axis of G = product of their strides positions;
+//   * every new dimension but the outermost is dense too (stride = its extent);
+//   * the outermost new dimension takes what is left of G, G / (inner new extents),
+//     which must divide, and the outermost old dimension's offset, counted in
+//     steps of the inner new extents (which must divide as well).
+// New dimensions of extent 1 left over in front get stride 1; old ones left over
+// in front must be dense.
+namespace {
+struct ReshapeRun {
+    int old_outer, old_inner;  // old dimensions [old_outer, old_inner]
+    int new_outer, new_inner;  // new dimensions [new_outer, new_inner]
+};
+}  // namespace
+
 static void reshape_view(const ModelTensorRef &in, const Dims &target, bool allowzero, Dims &shape,
                          Dims &strides, Dims &offsets) {
-    const Dims &os = in->shape(), &ost = in->strides(), &oof = in->offsets();
-    std::vector<DimType> ns;
-    if (target.ndims() == 0) {
-        ns.push_back(1);
-        if (os.nelems() != 1)
-            ARK_ERR(ModelError, "number of elements mismatch: reshape from ", os, " to ", target);
-    } else {
-        DimType total = 1;
-        for (int i = 0; i < target.ndims(); ++i) {
-            DimType d = target[i];
-            if (d == 0) d = allowzero ? 0 : os[i];
-            ns.push_back(d);
-            total *= d;
-        }
-        if (os.nelems() != total)
-            ARK_ERR(ModelError, "number of elements mismatch: reshape from ", os, " to ", target);
-    }
-    shape = Dims(ns);
-    std::ostringstream why;
-    why << "reshape failed as the strides of the input tensor is incompatible with the new shape. "
-           "A workaround is copying the input tensor to a new tensor, so that the data becomes "
-           "sequential in memory. Input shape "
-        << os << ", strides " << ost << ", new shape " << shape;
+    const Dims &old_shape = in->shape(), &old_strides = in->strides(), &old_offsets = in->offsets();
+    std::vector<DimType> want;
+    for (int i = 0; i < target.ndims(); ++i)
+        want.push_back((target[i] == 0 && !allowzero) ? old_shape[i] : target[i]);
+    if (want.empty()) want.push_back(1);  // a scalar is a one-element vector
+    shape = Dims(want);
+    if (shape.nelems() != old_shape.nelems())
+        ARK_ERR(ModelError, "reshape from ", old_shape, " to ", target, " changes the number of elements");
+    auto refuse = [&]() {
+        ARK_ERR(ModelError, "reshape of a tensor with shape ", old_shape, " and strides ", old_strides, " to ", shape,
+                " is not a view of the same memory (a dimension that would be merged is padded or offset); "
+                "copy the tensor into a dense one first");
+    };
+    auto dense = [&](int i) { return old_strides[i] == old_shape[i] && old_offsets[i] == 0; };
 
-    std::vector<DimType> rst, rof;  // innermost first
-    int oi = os.ndims() - 1, ni = shape.ndims() - 1;
-    DimType o_acc = os[oi], n_acc = shape[ni], st_acc = ost[oi], div = 1;
+    // cut both shapes into runs, innermost first
+    std::vector<ReshapeRun> runs;
+    int oi = old_shape.ndims() - 1, ni = shape.ndims() - 1;
     while (oi >= 0 && ni >= 0) {
-        if (o_acc == n_acc) {
-            if (st_acc % div != 0) ARK_ERR(ModelError, why.str());
-            DimType off = oof[oi];
-            for (int i = oi + 1; i < ost.ndims(); ++i) off *= ost[i];
-            for (DimType s : rst) off /= s;
-            rst.push_back(st_acc / div);
-            rof.push_back(off);
-            div = 1;
-            --ni;
-            --oi;
-            if (ni >= 0) n_acc = shape[ni];
-            if (oi >= 0) {
-                o_acc = os[oi];
-                st_acc = ost[oi];
-            }
-        } else if (o_acc > n_acc) {
-            div *= shape[ni];
-            rst.push_back(shape[ni]);
-            rof.push_back(0);
-            --ni;
-            if (ni >= 0) n_acc *= shape[ni];
-        } else {
-            if (ost[oi] != os[oi] || oof[oi] != 0) ARK_ERR(ModelError, why.str());
-            --oi;
-            if (oi >= 0) {
-                o_acc *= os[oi];
-                st_acc *= ost[oi];
+        ReshapeRun r{oi, oi, ni, ni};
+        DimType old_count = old_shape[oi], new_count = shape[ni];
+        bool open = true;
+        while (open) {
+            if (old_count == new_count) {
+                open = false;
+            } else if (old_count > new_count) {
+                if (r.new_outer == 0) break;
+                new_count *= shape[--r.new_outer];
+            } else {
+                if (r.old_outer == 0) break;
+                old_count *= old_shape[--r.old_outer];
             }
         }
+        if (open) refuse();  // cannot happen when the element counts agree
+        runs.push_back(r);
+        oi = r.old_outer - 1;
+        ni = r.new_outer - 1;
     }
-    while (ni >= 0 && shape[ni] == 1) {
-        rst.push_back(1);
-        rof.push_back(0);
-        --ni;
+    std::vector<DimType> new_strides((size_t)shape.ndims(), 1), new_offsets((size_t)shape.ndims(), 0);
+    for (const ReshapeRun &r : runs) {
+        DimType positions = 1, merged_inner = 1;  // G, and the extents of the old dimensions inside the outermost
+        for (int i = r.old_inner; i >= r.old_outer; --i) {
+            if (i > r.old_outer) {
+                if (!dense(i)) refuse();
+                merged_inner *= old_shape[i];
+            }
+            positions *= old_strides[i];
+        }
+        DimType split_inner = 1;
+        for (int j = r.new_inner; j > r.new_outer; --j) {
+            new_strides[(size_t)j] = shape[j];
+            split_inner *= shape[j];
+        }
+        if (split_inner == 0 || positions % split_inner != 0) refuse();
+        new_strides[(size_t)r.new_outer] = positions / split_inner;
+        // The outermost old dimension's offset, in elements of the run, must be a whole
+        // number of steps of the inner new extents: otherwise the view starts inside an
+        // inner new dimension and no (stride, offset) pair addresses it.  (The reference
+        // rounds down here and returns a view of the wrong elements.)
+        const DimType lead = old_offsets[r.old_outer] * merged_inner;
+        if (lead % split_inner != 0) refuse();
+        new_offsets[(size_t)r.new_outer] = lead / split_inner;
     }
-    while (oi >= 0 && os[oi] == 1) {
-        if (ost[oi] != os[oi] || oof[oi] != 0) ARK_ERR(ModelError, why.str());
-        --oi;
-    }
-    if (oi >= 0 || ni >= 0) ARK_ERR(ModelError, why.str());
-    strides = Dims(std::vector<DimType>(rst.rbegin(), rst.rend()));
-    offsets = Dims(std::vector<DimType>(rof.rbegin(), rof.rend()));
+    for (; ni >= 0; --ni)
+        if (shape[ni] != 1) refuse();
+    for (; oi >= 0; --oi)
+        if (old_shape[oi] != 1 || !dense(oi)) refuse();
+    strides = Dims(new_strides);
+    offsets = Dims(new_offsets);
 }
 
 // ark/ops/ops_reshape.cpp:153-204

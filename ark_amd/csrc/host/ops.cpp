@@ -108,16 +108,17 @@ static Json reference_config(const ModelOp &op, const Arch &arch) {
 // One slot of 8 waves (512 threads) per CU for every op, so a task always owns
 // the whole workgroup and s_barrier is the only intra-task barrier.
 constexpr int kWarps950 = 8;
-constexpr int kNumCu950 = 256;
 
 // Rows a wave takes per row-op task: one while that still gives every CU a task,
 // then more (up to 8), so a wave keeps the next row's loads in flight while it
 // reduces and stores the current one.
-static int64_t rows_per_wave950(int64_t rows) {
-    return std::max<int64_t>(1, std::min<int64_t>(8, rows / (kWarps950 * kNumCu950)));
+static int64_t rows_per_wave950(int64_t rows, int num_cu) {
+    return std::max<int64_t>(1, std::min<int64_t>(8, rows / ((int64_t)kWarps950 * num_cu)));
 }
 
-static Json rocm950_config(const ModelOp &op) {
+// `num_cu`: the processor count the plan is made for (the planner's NumProcessors
+// argument), which decides tile sizes, rows per wave and skinny-matmul task counts.
+static Json rocm950_config(const ModelOp &op, int num_cu) {
     const std::string &t = op.type();
     if (t == "Matmul") {
         auto dt = op.result_tensors()[0]->data_type();
@@ -139,7 +140,7 @@ static Json rocm950_config(const ModelOp &op) {
             Json tile = Json::array();
             tile.push_back(16); tile.push_back(256); tile.push_back(128);
             c["TileShapeMNK"] = tile;
-            c["NumTasks"] = (long long)gemv_default_tasks(rs[3], k, kNumCu950);
+            c["NumTasks"] = (long long)gemv_default_tasks(rs[3], k, num_cu);
             return c;
         }
         // Largest tile that divides the padded problem and still gives every CU
@@ -153,7 +154,7 @@ static Json rocm950_config(const ModelOp &op) {
             if ((trans_in || f32) && (c[0] != 128 || c[1] != 128)) continue;
             if (mnk[0] % c[0] || mnk[1] % c[1]) continue;
             tm = c[0]; tn = c[1];
-            if (batch * (mnk[0] / c[0]) * (mnk[1] / c[1]) >= kNumCu950) break;
+            if (batch * (mnk[0] / c[0]) * (mnk[1] / c[1]) >= num_cu) break;
         }
         if (tm == 0 || mnk[2] % 64 != 0)
             ARK_ERR(PlanError, "output padded shape MNK ", mnk,
@@ -180,7 +181,7 @@ static Json rocm950_config(const ModelOp &op) {
                                "64; got ", rs, ", dim ", k);
         const int64_t batch = rs[0] * rs[1];
         int64_t tm = 256;
-        if (rs[2] % 256 || batch * (rs[2] / 256) * (rs[3] / 128) < kNumCu950) tm = 128;
+        if (rs[2] % 256 || batch * (rs[2] / 256) * (rs[3] / 128) < num_cu) tm = 128;
         Json c = Json::object();
         c["NumWarps"] = kWarps950;
         c["SramBytes"] = gemm_lds_bytes((int)tm, 256);
@@ -201,7 +202,7 @@ static Json rocm950_config(const ModelOp &op) {
         int64_t outs = op.result_tensors()[0]->shape().nelems();
         // WarpWise: RowsPerWave output rows per wave; ElementWise: one output per thread
         if (last) {
-            const int64_t rpw = rows_per_wave950(outs);
+            const int64_t rpw = rows_per_wave950(outs, num_cu);
             c["RowsPerWave"] = (long long)rpw;
             c["NumTasks"] = (long long)div_up(outs, kWarps950 * rpw);
         } else {
@@ -226,7 +227,7 @@ static Json rocm950_config(const ModelOp &op) {
         c["SramBytes"] = 0;
         const Dims &s = op.result_tensors()[0]->shape();
         const int64_t rows = s.nelems() / s[-1];
-        const int64_t rpw = rows_per_wave950(rows);
+        const int64_t rpw = rows_per_wave950(rows, num_cu);
         // RMSNorm keeps its fp32 weights in LDS for the rows of a task
         if (t == "Rmsnorm" && op.read_tensors().size() > 1 &&
             op.read_tensors()[1]->data_type() == FP32.ref() && s[-1] * 4 <= 65536)
@@ -346,8 +347,8 @@ Json follower_config(const ModelOp &op, const Json &task_info) {
     return c;
 }
 
-Json default_config(const ModelOp &op, const Arch &arch) {
-    if (arch.belongs_to("ROCM_950")) return rocm950_config(op);
+Json default_config(const ModelOp &op, const Arch &arch, int num_processors) {
+    if (arch.belongs_to("ROCM_950")) return rocm950_config(op, std::max(1, num_processors));
     const std::string &t = op.type();
     if (t == "Softmax" || t == "Layernorm" || t == "Rmsnorm" || t == "Attention")
         ARK_ERR(PlanError, "op type ", t, " exists only on ROCM_950");

@@ -19,8 +19,9 @@ Dims matmul_problem_size(const Dims &in, const Dims &other, bool trans_in, bool 
 // Default plan config of a non-virtual op for an architecture: at least
 // NumWarps, SramBytes, NumTasks (ark/ops/ops_*.cpp default_config()).  For
 // CUDA_* / ROCM_90A / ROCM_942 the reference's rules are reproduced; ROCM_950
-// has this backend's own (one 8-wave slot per CU).
-Json default_config(const ModelOp &op, const Arch &arch);
+// has this backend's own (one 8-wave slot per CU), sized for the `num_processors`
+// the plan is made for.
+Json default_config(const ModelOp &op, const Arch &arch, int num_processors);
 
 // Config of an elementwise op that joins the task of `task_info` (an op fused
 // behind its producer by a PlannerContext with sync(false)) on ROCM_950: when

@@ -83,7 +83,7 @@ std::string Planner::Impl::plan(bool pretty) const {
             }
         }
         const bool config_given = !config.empty();
-        if (config.empty()) config = default_config(*op, arch_);
+        if (config.empty()) config = default_config(*op, arch_, num_processors_);
 
         Json ctx_id = node_ctx(node, "Id");
         Json ctx_sync = node_ctx(node, "Sync");

@@ -108,6 +108,17 @@ __device__ __forceinline__ float wave_allreduce(float v, Op op) {
     return v;
 }
 
+// ---- stores complete, then the workgroup meets ---------------------------------
+// A workgroup barrier alone does not wait for a wave's global stores: the compiler
+// emits no wait for a workgroup-scope release, and s_barrier does not drain the
+// memory counters.  Where one thread goes on to tell other workgroups that this
+// workgroup's data is in the L2 (an arrival atomic, a flag), every wave first waits
+// until its own stores are acknowledged (vmcnt counts loads and stores on gfx9) and
+// its LDS traffic is done, and only then joins the barrier.
+__device__ __forceinline__ void drain_stores_then_barrier() {
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ---- slot context -----------------------------------------------------------
 // A task runs on one "slot": a contiguous group of waves of the workgroup with
 // its own LDS window.  With one resident slot per CU (the gfx950 default) the

@@ -260,10 +260,10 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
             // Partials travel as agent-scope relaxed atomics (write-through
             // stores, L2-bypassing loads), so no cache-wide write-back or
             // invalidate is needed: those are serialised per L2 and cost more
-            // than the op itself when every task issues them.  Ordering: the
-            // workgroup barrier waits for the stores to complete, the counter
-            // is bumped after it, and the partials are read only after the
-            // counter has been seen full.
+            // than the op itself when every task issues them.  Ordering: every
+            // wave waits for its stores to be acknowledged (vmcnt 0) before the
+            // workgroup barrier, the counter is bumped after it, and the partials
+            // are read only after the counter has been seen full.
             const int t_first = (int)gemv_task_of((int64_t)nb * d.k_units, U, d.num_tasks);
             const int t_last = (int)gemv_task_of((int64_t)(nb + 1) * d.k_units - 1, U, d.num_tasks);
             const int parts = t_last - t_first + 1;
@@ -275,8 +275,7 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
                     __hip_atomic_store(Pb + ((int64_t)(task - t_first) * d.m + m) * kGemvCols + n_local,
                                        sums[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-            s.sync();
+            drain_stores_then_barrier();
             if (tid == 0) {
                 const unsigned prev = __hip_atomic_fetch_add(d.counters + nb, 1u, __ATOMIC_RELAXED,
                                                              __HIP_MEMORY_SCOPE_AGENT);

@@ -30,7 +30,8 @@ __device__ __forceinline__ bool in_range(int x, int b, int e, int s) {
 static __device__ bool grid_barrier(GridBarrier *bar, unsigned nblocks, LoopControl *ctl,
                              uint64_t limit_ticks) {
     int *lds_flag = reinterpret_cast<int *>(g_loop_lds);
-    __syncthreads();
+    // every wave's stores are acknowledged by the L2 before thread 0 writes the L2 back
+    drain_stores_then_barrier();
     if (threadIdx.x == 0) {
         int ok = 1;
         if (nblocks > 1) {
@@ -119,9 +120,10 @@ static __device__ bool poll_reached(unsigned *word, unsigned target, LoopControl
 static __device__ bool grid_barrier_xcd(LoopControl *ctl, XcdInfo &xi, uint64_t limit_ticks) {
     int *lds_flag = reinterpret_cast<int *>(g_loop_lds);
     xi.epoch += 1u;
-    // workgroup barrier with a workgroup-scope release: every wave has waited
-    // for its stores to be acknowledged by the L2
-    __syncthreads();
+    // every wave waits until the L2 has acknowledged its stores, then the workgroup
+    // meets: the arrival below may be what lets the XCD's last arriver write the L2
+    // back, and a store still in flight then would stay dirty in this L2 only
+    drain_stores_then_barrier();
     if (threadIdx.x == 0) {
         GridBarrier *xb = &ctl->xcd[xi.x];
         const unsigned prev = __hip_atomic_fetch_add(&xb->count, 1u, __ATOMIC_RELAXED, AGENT);
@@ -401,7 +403,9 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(
             if (ok) ok = run_body<FAM>(prog, ctl, xi, wait_ticks);
         }
         if (!ok) break;
-        // results must be visible to the host before the command is cleared
+        // results must be visible to the host before the command is cleared: every
+        // wave's stores are in the L2 before thread 0's system-scope release
+        drain_stores_then_barrier();
         if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
         if (!grid_barrier_xcd(ctl, xi, wait_ticks)) break;
         if (one_shot_iters > 0) return;

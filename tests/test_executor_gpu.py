@@ -652,3 +652,100 @@ def test_fused_ops_with_different_task_counts_are_refused():
     with pytest.raises(ArkmiError) as e:
         Executor(m.plan(device_id=0), device_id=0).compile()
     assert e.value.kind == "PlanError" and "NumTasks" in str(e.value)
+
+
+# ---------------------------------------------------------------- barriers that must stay
+@pytest.mark.parametrize("n", [1024, 4096])
+def test_gemm_feeding_gemm_keeps_grid_barrier(oracle, n):
+    """(X @ W1) @ W2 with square operands: both GEMMs cut equal output shapes into the same tiles on
+    the same workgroups and Y1 is seen through one view, but task t of the second GEMM reads a whole
+    row panel of Y1, written by other workgroups on other L2s.  The barrier between them must stay a
+    grid barrier.  Checked on sampled rows against the oracle."""
+    from ark_amd import Model
+    dtype = "fp16"
+    x = make(oracle, (n, n), dtype, 81, "uniform")
+    w1 = make(oracle, (n, n), dtype, 82, "normal", scale=1.0 / np.sqrt(n))
+    w2 = make(oracle, (n, n), dtype, 83, "normal", scale=1.0 / np.sqrt(n))
+    m = Model()
+    tx, t1, t2 = (m.tensor([n, n], dtype) for _ in range(3))
+    y2 = m.matmul(m.matmul(tx, t1), t2)
+    (got,), ex, _ = run_model(m, {tx: x, t1: w1, t2: w2}, [y2], iters=2)
+    info = ex.info()
+    assert info["barriers_local"] == 0 and info["barriers_elided"] == 0, info
+    pick = np.sort(np.random.default_rng(3).choice(n, 16, replace=False))
+    pick[0], pick[-1] = 0, n - 1
+    y1 = oracle.matmul(np.ascontiguousarray(x[pick]), w1, dtype)
+    close(oracle, oracle.matmul(y1, w2, dtype), got[pick], dtype, 1e-2)
+
+
+def test_iterated_gemm_plus_one_keeps_iteration_barrier(oracle, monkeypatch):
+    """X <- (X @ W) * 0.5 + ... in place across iterations: the next iteration's GEMM reads row
+    panels of X that other workgroups' elementwise tasks wrote, so iterations stay separated by the
+    grid barrier even though the add rides on the GEMM's tiles."""
+    from ark_amd import Model
+    monkeypatch.setenv("ARKMI_ITERATION_BARRIER", "0")
+    dtype, n = "fp16", 512
+    x = make(oracle, (n, n), dtype, 84, "uniform")
+    w = make(oracle, (n, n), dtype, 85, "normal", scale=1.0 / np.sqrt(n))
+    m = Model()
+    tx, tw = m.tensor([n, n], dtype), m.tensor([n, n], dtype)
+    y = m.matmul(tx, tw)
+    m.add(y, 1.0, tx)
+    iters = 4
+    (got,), ex, _ = run_model(m, {tx: x, tw: w}, [tx], iters=iters)
+    assert ex.info()["iteration_sync"] == 2, ex.info()
+    want = x
+    for _ in range(iters):
+        want = oracle.scalar(oracle.matmul(want, w, dtype), 1.0, "add", dtype)
+    # four rounds of rounding in different summation orders: judged against the largest value
+    t, g = (oracle.to_f32(a, dtype).astype(np.float64) for a in (want, got))
+    assert np.abs(t - g).max() <= 1e-2 * np.abs(t).max()
+
+
+def _chain_graphs():
+    """Small multi-op graphs whose dependencies cross workgroups in different ways."""
+    def gemm_gemm(m, dt):
+        a, b, c = m.tensor([512, 512], dt), m.tensor([512, 512], dt), m.tensor([512, 512], dt)
+        return [a, b, c], [m.matmul(m.matmul(a, b), c)]
+
+    def ewise_gemm(m, dt):
+        a, b = m.tensor([512, 512], dt), m.tensor([512, 512], dt)
+        return [a, b], [m.matmul(m.mul(a, 0.5), b)]
+
+    def gemm_reduce(m, dt):
+        a, b = m.tensor([512, 256], dt), m.tensor([256, 512], dt)
+        y = m.matmul(a, b)
+        return [a, b], [m.reduce_sum(y, -1), m.softmax(y)]
+
+    def gemm_ewise_transpose(m, dt):
+        a, b = m.tensor([256, 256], dt), m.tensor([256, 256], dt)
+        y = m.relu(m.matmul(a, b))
+        return [a, b], [m.transpose(y, [1, 0]), m.add(y, y)]
+
+    def rows_then_gemm(m, dt):
+        a, b = m.tensor([256, 512], dt), m.tensor([512, 256], dt)
+        return [a, b], [m.matmul(m.softmax(a), b)]
+
+    return {"gemm_gemm": gemm_gemm, "ewise_gemm": ewise_gemm, "gemm_reduce": gemm_reduce,
+            "gemm_ewise_transpose": gemm_ewise_transpose, "rows_then_gemm": rows_then_gemm}
+
+
+@pytest.mark.parametrize("graph", sorted(_chain_graphs()))
+def test_elided_barriers_give_the_reference_placements_results(oracle, graph, monkeypatch):
+    """Each graph runs twice, with the barriers this backend keeps and with every barrier the
+    reference places (ARKMI_KEEP_ALL_BARRIERS=1): outputs must agree bit for bit, over several
+    iterations."""
+    from ark_amd import Model
+    dtype = "fp16"
+    outs = []
+    for keep in ("1", "0"):
+        monkeypatch.setenv("ARKMI_KEEP_ALL_BARRIERS", keep)
+        m = Model()
+        ins, fetch = _chain_graphs()[graph](m, dtype)
+        feeds = {t: make(oracle, tuple(t.shape), dtype, 90 + i, "uniform", -0.25, 0.25) for i, t in enumerate(ins)}
+        got, ex, _ = run_model(m, feeds, fetch, iters=3)
+        if keep == "1":
+            assert ex.info()["barriers_elided"] == 0 and ex.info()["barriers_local"] == 0
+        outs.append(got)
+    for a, b in zip(*outs):
+        assert np.array_equal(a, b), graph

@@ -122,3 +122,55 @@ def test_gemv_in_loop_kernel(oracle, dtype, m):
     ex.stop()
     ref = oracle.matmul(x, w, dtype)
     _check(oracle, ref, got, dtype, 4.0 * 0.25, k)
+
+
+def _sampled_columns_check(oracle, x, w, got, dtype, cols):
+    """Oracle on sampled output columns (all rows of X against those columns of W)."""
+    ref = oracle.matmul(x, np.ascontiguousarray(w[:, cols]), dtype)
+    _check(oracle, ref, np.ascontiguousarray(got[:, cols]), dtype, 4.0 * 0.25, x.shape[1])
+
+
+@pytest.mark.parametrize("m", [1, 8])
+@pytest.mark.parametrize("n,k", [(12288, 4096), (22016, 4096), (4096, 4096)])
+def test_gemv_decode_projection_shapes(oracle, m, n, k):
+    """The remaining Llama-2-7B decode shapes (W_qkv, W_gate/up, W_o; W_down is in test_gemv_shapes),
+    bf16, batch 1 and 8; the oracle evaluates 512 sampled columns plus the first and last."""
+    from ark_amd import ops
+    dtype = "bf16"
+    x = make(oracle, (m, k), dtype, seed=31, dist="normal")
+    w = make(oracle, (k, n), dtype, seed=32, dist="normal", scale=0.02)
+    got = to_np(ops.gemv(to_gpu(x, dtype), to_gpu(w, dtype)), dtype)
+    cols = np.sort(np.random.default_rng(4).choice(n, 512, replace=False))
+    cols[0], cols[-1] = 0, n - 1
+    _sampled_columns_check(oracle, x, w, got, dtype, cols)
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+def test_decode_step_four_projections_in_one_plan(oracle, batch):
+    """The decode step the benchmark times: x[B,4096] against W_qkv[4096,12288], W_o[4096,4096],
+    W_gate/up[4096,22016] and x2[B,11008] against W_down[11008,4096], bf16, as four skinny matmuls of
+    one plan in the loop kernel, three iterations.  All four outputs against the oracle on sampled
+    columns (512 per matrix)."""
+    from ark_amd import Model, Executor
+    dtype = "bf16"
+    shapes = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
+    mod = Model()
+    xs, ws, ys, vals = [], [], [], {}
+    for i, (k, n) in enumerate(shapes):
+        tx, tw = mod.tensor([batch, k], dtype), mod.tensor([k, n], dtype)
+        vals[tx] = make(oracle, (batch, k), dtype, seed=40 + i, dist="normal")
+        vals[tw] = make(oracle, (k, n), dtype, seed=50 + i, dist="normal", scale=0.02)
+        xs.append(tx); ws.append(tw); ys.append(mod.matmul(tx, tw))
+    ex = Executor(mod.plan(device_id=0)).compile()
+    assert ex.info()["kernel_families"] == 8
+    for t, a in vals.items():
+        ex.tensor_write(t, a)
+    ex.launch()
+    ex.run(3)
+    ex.wait()
+    got = [ex.tensor_read(t) for t in ys]
+    ex.stop()
+    for (k, n), tx, tw, g in zip(shapes, xs, ws, got):
+        cols = np.sort(np.random.default_rng(n).choice(n, 512, replace=False))
+        cols[0], cols[-1] = 0, n - 1
+        _sampled_columns_check(oracle, vals[tx], vals[tw], g, dtype, cols)

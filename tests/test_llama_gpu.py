@@ -60,16 +60,18 @@ def test_ffn_small(oracle, dtype):
     assert mx <= TOL and rms <= TOL, (mx, rms)
 
 
-def test_ffn_full_size_sampled_rows(oracle):
-    """x[8192,4096] bf16 -> 11008 -> 4096 in one loop kernel; the oracle
-    evaluates 48 sampled rows (every output column of those rows)."""
+@pytest.mark.parametrize("fused", [False, True])
+def test_ffn_full_size_sampled_rows(oracle, fused):
+    """x[8192,4096] bf16 -> 11008 -> 4096 in one loop kernel, as the reference's
+    composition and as the fused path the benchmark times (SwiGLU as one GEMM pass);
+    the oracle evaluates 48 sampled rows (every output column of those rows)."""
     from ark_amd import Model, llama
     dtype, rows, dim, hidden = "bf16", 8192, 4096, 11008
     x, w1, w2, w3 = _ffn_case(oracle, rows, dim, hidden, dtype, 200)
     m = Model()
     tx = m.tensor([rows, dim], dtype)
     ff = llama.FeedForward(m, dim, hidden, dtype)
-    out = ff.forward(tx)
+    out = ff.forward(tx, fused=fused)
     got, info = _run(m, {tx: x, ff.w1: w1, ff.w2: w2, ff.w3: w3}, out)
     pick = np.sort(np.random.default_rng(7).choice(rows, 48, replace=False))
     pick[0], pick[-1] = 0, rows - 1

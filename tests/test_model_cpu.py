@@ -136,6 +136,67 @@ def test_reshape_stride_inference():
     raises_model_error(lambda: m.reshape(p, [24]))
 
 
+def _addresses(shape, strides, offsets):
+    """Element offsets of a view inside its buffer, in row-major order of `shape`."""
+    import itertools
+    import numpy as np
+    pitch = [1] * len(shape)
+    for i in range(len(shape) - 2, -1, -1):
+        pitch[i] = pitch[i + 1] * strides[i + 1]
+    out = []
+    for idx in itertools.product(*[range(s) for s in shape]):
+        out.append(sum((o + i) * p for i, o, p in zip(idx, offsets, pitch)))
+    return np.array(out, dtype=np.int64)
+
+
+def test_reshape_addresses_the_same_elements_brute_force():
+    """Whatever strides/offsets reshape infers, element i (row-major) of the result must
+    sit where element i of the input sits: brute force over random padded and offset
+    views and every factorisation of their element count into up to four extents.  A
+    refusal is allowed only when a merged dimension is padded or offset."""
+    import itertools
+    import numpy as np
+    rng = np.random.default_rng(7)
+
+    def factorisations(n, k):
+        if k == 1:
+            yield [n]
+            return
+        for d in range(1, n + 1):
+            if n % d == 0:
+                for rest in factorisations(n // d, k - 1):
+                    yield [d] + rest
+
+    m = Model()
+    accepted = refused = 0
+    for trial in range(60):
+        nd = int(rng.integers(1, 5))
+        shape = [int(rng.choice([1, 2, 3, 4, 6])) for _ in range(nd)]
+        pad = [int(rng.choice([0, 0, 1, 2])) for _ in range(nd)]
+        offs = [int(rng.integers(0, p + 1)) for p in pad]
+        strides = [s + p for s, p in zip(shape, pad)]
+        t = m.tensor(shape, "fp32", strides=strides, offsets=offs)
+        src = _addresses(shape, strides, offs)
+        n = int(np.prod(shape))
+        dense_all = all(p == 0 for p in pad)
+        for k in range(1, 5):
+            for target in itertools.islice(factorisations(n, k), 12):
+                try:
+                    r = m.reshape(t, target)
+                except ArkmiError as e:
+                    assert e.kind == "ModelError"
+                    assert not dense_all, (shape, strides, offs, target)  # a dense tensor reshapes to anything
+                    refused += 1
+                    continue
+                accepted += 1
+                assert r.shape == target
+                for sh, st, of in zip(r.shape, r.strides, r.offsets):
+                    assert of + sh <= st
+                dst = _addresses(r.shape, r.strides, r.offsets)
+                assert np.array_equal(src, dst), (shape, strides, offs, target, r.strides, r.offsets)
+    assert accepted > 300 and refused > 50, (accepted, refused)
+
+
 def test_refer_and_cast_views():
     m = Model()
     t = m.tensor([4, 8], "fp16")
