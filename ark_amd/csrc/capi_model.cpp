@@ -94,6 +94,31 @@ int arkmi_model_create(int rank, int world_size, arkmi_model **out) {
     });
 }
 
+int arkmi_model_from_json(const char *model_json, arkmi_model **out) {
+    return guard_ark([&] {
+        if (!model_json || !out) ARKMI_FAIL(ARKMI_INVALID_USAGE, "null argument");
+        Json j;
+        try {
+            j = Json::parse(model_json);
+        } catch (const std::exception &e) {
+            ARK_ERR(ModelError, "failed to parse the model: ", e.what());
+        }
+        auto graph = ark::ModelGraph::Impl::deserialize(j);  // verifies the format first
+        auto m = std::make_unique<arkmi_model>(graph->rank_, graph->world_size_);
+        // every tensor of the file becomes addressable by its id, and ids handed out
+        // later (ops added to the rebuilt model) stay clear of the file's
+        for (const auto &node : graph->nodes_)
+            for (const auto *vec : {&node->op->read_tensors(), &node->op->write_tensors(), &node->op->result_tensors()})
+                for (const auto &t : *vec) {
+                    m->tensors[(int64_t)t->id()] = ark::Tensor(t);
+                    ark::ModelTensor::reserve_id(t->id());
+                    ark::ModelBuffer::reserve_id(t->buffer()->id());
+                }
+        ark::ModelGraphAccess::adopt(m->model, std::move(graph));
+        *out = m.release();
+    });
+}
+
 int arkmi_model_destroy(arkmi_model *m) {
     return guard_ark([&] {
         if (!m) return;

@@ -232,6 +232,67 @@ extern "C" int arkmi_gemv_plan(int m, int n, int k, int num_tasks, int *num_task
     });
 }
 
+namespace arkmi {
+
+// Validates the arguments of a skinny matmul, fills the descriptor and launches it with
+// `workspace` (counters first, then partials) of at least the planned size.
+static void launch_gemv(int dtype, const void *x, const void *w, void *y, int m, int n, int k, int64_t ldx,
+                        int64_t ldw, int64_t ldy, int num_tasks, void *workspace, hipStream_t st) {
+    if (!x || !w || !y) ARKMI_FAIL(ARKMI_INVALID_USAGE, "null tensor pointer");
+    if (ldx < k || ldw < n || ldy < n) ARKMI_FAIL(ARKMI_INVALID_USAGE, "leading dimension too small");
+    if ((n % 8) || (ldx % 8) || (ldw % 8) || ((uintptr_t)x & 15) || ((uintptr_t)w & 15))
+        ARKMI_FAIL(ARKMI_UNSUPPORTED, "operands must be 16-byte aligned with N and leading dimensions % 8 == 0");
+    GemvDesc d{};
+    d.x = x; d.w = w; d.y = y;
+    d.m = m; d.n = n; d.k = k;
+    d.ldx = (int)ldx; d.ldw = (int)ldw; d.ldy = (int)ldy;
+    d.dtype = dtype;
+    gemv_partition(d, num_tasks);
+    d.counters = static_cast<unsigned int *>(workspace);
+    d.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + gemv_counter_bytes(d.n_blocks));
+    static bool attr_set[2] = {false, false};
+    const int ti = dtype == ARKMI_FP16 ? 0 : 1;
+    const void *kern = ti == 0 ? (const void *)gemv_kernel<f16> : (const void *)gemv_kernel<bf16>;
+    if (!attr_set[ti]) {
+        ARKMI_HIP(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kGemvLdsBytes));
+        attr_set[ti] = true;
+    }
+    int ntasks = d.num_tasks;
+    void *args[] = {&d, &ntasks};
+    ARKMI_HIP(hipLaunchKernel(kern, dim3(ntasks), dim3(kBlock), args, kGemvLdsBytes, st));
+}
+
+// ---- the skinny matmul with its workspace inside the library ------------------------
+// Device memory that belongs to the code object: every GPU the library runs on holds its
+// own copy at its own address until the process ends.  In host code the array's name is a
+// stand-in, not a device address; the address of a device's copy comes from
+// hipGetSymbolAddress with that device current, once per device.
+constexpr size_t kGemvStaticBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char g_gemv_scratch[kGemvStaticBytes];
+
+constexpr int kMaxDevices = 64;
+static void *g_gemv_scratch_ptr[kMaxDevices];  // per device, null until resolved
+
+static void *gemv_static_workspace() {
+    const int dev = current_device();
+    if (dev < 0 || dev >= kMaxDevices) ARKMI_FAIL(ARKMI_UNSUPPORTED, "device index ", dev, " out of range");
+    if (!g_gemv_scratch_ptr[dev]) {
+        void *p = nullptr;
+        ARKMI_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_gemv_scratch)));
+        if (!p) ARKMI_FAIL(ARKMI_GPU_ERROR, "the library's static workspace has no address on device ", dev);
+        g_gemv_scratch_ptr[dev] = p;
+    }
+    return g_gemv_scratch_ptr[dev];
+}
+
+// Zero fill by a kernel: callers may be under stream capture, where memset nodes are avoided.
+__global__ void zero_words_kernel(unsigned int *p, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+}  // namespace arkmi
+
 extern "C" int arkmi_gemv(int dtype, const void *x, const void *w, void *y, int m, int n, int k,
                           int64_t ldx, int64_t ldw, int64_t ldy, int num_tasks, void *workspace,
                           size_t workspace_bytes, void *stream) {
@@ -241,32 +302,32 @@ extern "C" int arkmi_gemv(int dtype, const void *x, const void *w, void *y, int 
         size_t need = 0;
         if (int rc = arkmi_gemv_plan(m, n, k, num_tasks, &num_tasks, &need))
             throw Error(rc, arkmi_last_error());
-        if (!x || !w || !y) ARKMI_FAIL(ARKMI_INVALID_USAGE, "null tensor pointer");
-        if (ldx < k || ldw < n || ldy < n) ARKMI_FAIL(ARKMI_INVALID_USAGE, "leading dimension too small");
-        if ((n % 8) || (ldx % 8) || (ldw % 8) || ((uintptr_t)x & 15) || ((uintptr_t)w & 15))
-            ARKMI_FAIL(ARKMI_UNSUPPORTED,
-                       "operands must be 16-byte aligned with N and leading dimensions % 8 == 0");
         if (!workspace || workspace_bytes < need)
             ARKMI_FAIL(ARKMI_INVALID_USAGE, "workspace of ", need, " bytes needed, got ", workspace_bytes);
-        GemvDesc d{};
-        d.x = x; d.w = w; d.y = y;
-        d.m = m; d.n = n; d.k = k;
-        d.ldx = (int)ldx; d.ldw = (int)ldw; d.ldy = (int)ldy;
-        d.dtype = dtype;
-        gemv_partition(d, num_tasks);
-        d.counters = static_cast<unsigned int *>(workspace);
-        d.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) +
-                                              gemv_counter_bytes(d.n_blocks));
+        launch_gemv(dtype, x, w, y, m, n, k, ldx, ldw, ldy, num_tasks, workspace, (hipStream_t)stream);
+    });
+}
+
+extern "C" size_t arkmi_gemv_static_limit(void) { return arkmi::kGemvStaticBytes; }
+
+extern "C" int arkmi_gemv_static(int dtype, const void *x, const void *w, void *y, int m, int n, int k,
+                                 int64_t ldx, int64_t ldw, int64_t ldy, int num_tasks, void *stream) {
+    return guard([&] {
+        if (dtype != ARKMI_FP16 && dtype != ARKMI_BF16)
+            ARKMI_FAIL(ARKMI_UNSUPPORTED, "the skinny matmul supports fp16/bf16, got dtype ", dtype);
+        size_t need = 0;
+        if (int rc = arkmi_gemv_plan(m, n, k, num_tasks, &num_tasks, &need))
+            throw Error(rc, arkmi_last_error());
+        if (need > kGemvStaticBytes)
+            ARKMI_FAIL(ARKMI_UNSUPPORTED, "this shape needs ", need, " bytes of workspace; the library's static workspace holds ",
+                       kGemvStaticBytes, " (use arkmi_gemv with a workspace of your own)");
+        void *ws = gemv_static_workspace();
         hipStream_t st = (hipStream_t)stream;
-        static bool attr_set[2] = {false, false};
-        const int ti = dtype == ARKMI_FP16 ? 0 : 1;
-        const void *kern = ti == 0 ? (const void *)gemv_kernel<f16> : (const void *)gemv_kernel<bf16>;
-        if (!attr_set[ti]) {
-            ARKMI_HIP(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kGemvLdsBytes));
-            attr_set[ti] = true;
-        }
-        int ntasks = d.num_tasks;
-        void *args[] = {&d, &ntasks};
-        ARKMI_HIP(hipLaunchKernel(kern, dim3(ntasks), dim3(kBlock), args, kGemvLdsBytes, st));
+        // the array keeps whatever the last call left: the arrival counters must start at zero
+        const int n_blocks = (n + kGemvCols - 1) / kGemvCols;
+        const int words = (int)(gemv_counter_bytes(n_blocks) / 4);
+        hipLaunchKernelGGL(zero_words_kernel, dim3((words + 255) / 256), dim3(256), 0, st, static_cast<unsigned int *>(ws), words);
+        ARKMI_HIP(hipGetLastError());
+        launch_gemv(dtype, x, w, y, m, n, k, ldx, ldw, ldy, num_tasks, ws, st);
     });
 }

@@ -201,6 +201,7 @@ static size_t g_next_tensor_id = 0;
 
 ModelBuffer::ModelBuffer(int rank) : id_(g_next_buffer_id++), rank_(rank) {}
 void ModelBuffer::reset_ids(size_t next) { g_next_buffer_id = next; }
+void ModelBuffer::reserve_id(size_t id) { g_next_buffer_id = std::max(g_next_buffer_id, id + 1); }
 
 Json ModelBuffer::serialize() const {
     Json j = Json::object();
@@ -271,6 +272,7 @@ ModelTensor::ModelTensor(const ModelTensor &o)
       strides_(o.strides_), offsets_(o.offsets_), padded_shape_(o.padded_shape_) {}
 
 void ModelTensor::reset_ids(size_t next) { g_next_tensor_id = next; }
+void ModelTensor::reserve_id(size_t id) { g_next_tensor_id = std::max(g_next_tensor_id, id + 1); }
 
 size_t ModelTensor::shape_bytes() const { return shape_.nelems() * data_type_->bytes(); }
 

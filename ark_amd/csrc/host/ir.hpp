@@ -105,6 +105,8 @@ class ModelBuffer {
     static std::shared_ptr<ModelBuffer> deserialize(const Json &j);
     // Process-global id counter; tests reset it to reproduce golden files.
     static void reset_ids(size_t next = 0);
+    // Moves the counter past `id` (ids read from a file must not be handed out again).
+    static void reserve_id(size_t id);
 
    private:
     size_t id_;
@@ -135,6 +137,7 @@ class ModelTensor {
     Json serialize() const;
     static std::shared_ptr<ModelTensor> deserialize(const Json &j);
     static void reset_ids(size_t next = 0);
+    static void reserve_id(size_t id);
 
    private:
     size_t id_;

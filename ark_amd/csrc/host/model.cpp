@@ -748,6 +748,7 @@ class Context::Impl {
 
 std::shared_ptr<ContextStack> ModelGraphAccess::context(Model &model) { return model.impl_->context_; }
 ModelGraph::Impl &ModelGraphAccess::impl(const ModelGraph &g) { return *g.impl_; }
+void ModelGraphAccess::adopt(ModelGraph &g, std::unique_ptr<ModelGraph::Impl> impl) { g.impl_ = std::move(impl); }
 
 Context::Context(Model &model) : impl_(std::make_shared<Impl>(model)) {}
 int Context::id() const { return impl_->id_; }

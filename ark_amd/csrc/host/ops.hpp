@@ -11,6 +11,8 @@ namespace ark {
 struct ModelGraphAccess {
     static std::shared_ptr<ContextStack> context(Model &model);
     static ModelGraph::Impl &impl(const ModelGraph &g);
+    // Replaces the graph of `g` (a model rebuilt from its serialized form).
+    static void adopt(ModelGraph &g, std::unique_ptr<ModelGraph::Impl> impl);
 };
 
 Dims broadcast_shape(const Dims &a, const Dims &b);

@@ -105,6 +105,18 @@ class Model:
         check(lib().arkmi_model_create(ctypes.c_int(rank), ctypes.c_int(world_size),
                                        ctypes.byref(self._h)))
 
+    @classmethod
+    def from_json(cls, text):
+        """A model rebuilt from the text Model.serialize() writes (the reference's model
+        file, docs/model_file.md); tensors keep the ids of the file."""
+        self = cls.__new__(cls)
+        self._h = ctypes.c_void_p()
+        check(lib().arkmi_model_from_json(text.encode(), ctypes.byref(self._h)))
+        return self
+
+    def tensor_by_id(self, tid):
+        return Tensor(self, tid)
+
     def __del__(self):
         if getattr(self, "_h", None):
             lib().arkmi_model_destroy(self._h)

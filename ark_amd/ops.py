@@ -163,3 +163,30 @@ def gemv(x, w, out=None, num_tasks=0):
         ctypes.c_int64(o2.stride(0)), ctypes.c_int(ntasks.value), _ptr(ws),
         ctypes.c_size_t(need.value), _stream()))
     return out.reshape(n) if x.dim() == 1 and out.dim() == 2 and out.shape[0] == 1 else out
+
+
+def gemv_static(x, w, out, num_tasks=0):
+    """gemv() through the entry point that allocates nothing: the workspace is a fixed array inside
+    the library (arkmi_gemv_static_limit() bytes per GPU) and `out` must be given.  Calls on one GPU
+    share that array and must not overlap in time."""
+    _require_cuda(x, w, out)
+    if x.dtype != w.dtype:
+        raise TypeError("operand dtypes differ")
+    x2 = x.reshape(1, -1) if x.dim() == 1 else x
+    m, k = x2.shape
+    if w.shape[0] != k:
+        raise ValueError(f"inner dimensions differ: {tuple(x.shape)} x {tuple(w.shape)}")
+    n = w.shape[1]
+    if x2.stride(-1) != 1 or w.stride(-1) != 1:
+        raise ValueError("innermost axis must be dense")
+    o2 = out.reshape(m, n)
+    check(lib().arkmi_gemv_static(
+        ctypes.c_int(_dt(x2)), _ptr(x2), _ptr(w), _ptr(o2), ctypes.c_int(m), ctypes.c_int(n),
+        ctypes.c_int(k), ctypes.c_int64(x2.stride(0)), ctypes.c_int64(w.stride(0)),
+        ctypes.c_int64(o2.stride(0)), ctypes.c_int(num_tasks), _stream()))
+    return out
+
+
+def gemv_static_limit():
+    lib().arkmi_gemv_static_limit.restype = ctypes.c_size_t
+    return int(lib().arkmi_gemv_static_limit())

@@ -151,6 +151,13 @@ void arkmi_free(void *p);
 void arkmi_reset_ids(void);
 
 int arkmi_model_create(int rank, int world_size, arkmi_model **out);
+/* A model rebuilt from its serialized form: the text ark::Model::serialize()
+ * writes (schema ark/model/model_json.cpp:24-101, docs/model_file.md; written by
+ * ark/model/model_graph_impl.cpp:318-345).  This is how a caller that keeps the
+ * reference's own ark::Model hands a finished graph to this library's planner:
+ * arkmi_model_from_json(model.serialize()) -> arkmi_model_plan().  Tensors keep the
+ * ids of the file; a malformed file is ARKMI_MODEL_ERROR. */
+int arkmi_model_from_json(const char *model_json, arkmi_model **out);
 int arkmi_model_destroy(arkmi_model *m);
 /* Model::tensor.  Optional arrays may be NULL. */
 int arkmi_model_tensor(arkmi_model *m, int ndims, const int64_t *shape,

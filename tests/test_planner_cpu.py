@@ -62,6 +62,33 @@ def test_model_json_golden_byte_for_byte():
     assert names == ["matmul", "sigmoid", "mul", "matmul_1", "mul_1", "matmul_2"]
 
 
+def test_model_file_round_trip_plans_like_the_model_that_wrote_it():
+    """The reference's model file is the hand-over format at the boundary: model.json (written by
+    ark::Model::serialize, examples/tutorial/model.json) read back through arkmi_model_from_json
+    serializes to the same bytes and plans to default_plan.json byte for byte."""
+    from ark_amd import Model, ArkmiError
+    m = Model.from_json(gold("model.json"))
+    assert m.serialize() == gold("model.json")
+    assert strip_arch(m.plan(arch="CUDA_80", num_processors=108)) == gold("default_plan.json")
+    # tensors of the file are addressable by id, and new ops do not reuse ids of the file
+    j = json.loads(gold("model.json"))
+    ids = {t["Id"] for n in j["Nodes"] for k in ("ReadTensors", "WriteTensors", "ResultTensors") for t in n["Op"][k]}
+    last = m.tensor_by_id(max(ids))
+    assert last.shape == [1, 512, 4096] and last.dtype == "fp16"
+    extra = m.relu(last)
+    assert extra.id not in ids and extra.buffer_id not in {
+        t["Buffer"]["Id"] for n in j["Nodes"] for k in ("ReadTensors", "WriteTensors", "ResultTensors") for t in n["Op"][k]}
+    # the same file planned for this backend's architecture: the gfx950 rules apply
+    m2 = Model.from_json(gold("model.json"))
+    p950 = json.loads(m2.plan(arch="ROCM_950", num_processors=256))
+    assert p950["Architecture"] == "ROCM_950" and p950["NumWarpsPerProcessor"] == 8
+    # malformed files are model errors
+    for bad in ("{", "{}", json.dumps({"Rank": 0, "WorldSize": 1, "Nodes": [{"Id": 0}]})):
+        with pytest.raises(ArkmiError) as e:
+            Model.from_json(bad)
+        assert e.value.kind == "ModelError", bad
+
+
 def test_plan_oracle_reproduces_golden():
     m = ffn_model()
     model = m.dump(compressed=True, with_context=True)
