@@ -122,6 +122,21 @@ int arkmi_gemv(int dtype, const void *x, const void *w, void *y, int m, int n,
                int k, int64_t ldx, int64_t ldw, int64_t ldy, int num_tasks,
                void *workspace, size_t workspace_bytes, void *stream);
 
+/* arkmi_gemv for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments and results as arkmi_gemv, bit for
+ * bit, without the workspace: the split-K partial sums and arrival counters live in
+ * a fixed array inside the library (arkmi_gemv_static_limit() bytes, 16 MiB, held by
+ * every GPU the library runs on until the process ends).  The call allocates and
+ * frees nothing; it launches one small kernel that zeroes the counters and then the
+ * matmul, both on `stream`.  A shape whose workspace (arkmi_gemv_plan) exceeds the
+ * array is refused with ARKMI_UNSUPPORTED.  All calls on one GPU share the array:
+ * calls that overlap in time on one GPU race. */
+size_t arkmi_gemv_static_limit(void);
+int arkmi_gemv_static(int dtype, const void *x, const void *w, void *y, int m, int n,
+                      int k, int64_t ldx, int64_t ldw, int64_t ldy, int num_tasks,
+                      void *stream);
+
 /* ------------------------------------------------------------------------
  * Model building and planning for bindings that cannot use the C++ classes
  * directly.  Every call maps onto one member of ark::Model / PlannerContext /

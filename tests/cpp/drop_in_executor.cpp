@@ -72,6 +72,7 @@ int main() {
         }};
     ark::DefaultExecutor exe(m, 0, nullptr, rules);
     EXPECT(rule_calls == 2);
+    exe.compile();
     exe.tensor_write(ta, ah);
     exe.tensor_write(tb, bh);
     exe.launch();

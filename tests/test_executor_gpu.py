@@ -675,7 +675,12 @@ def test_gemm_feeding_gemm_keeps_grid_barrier(oracle, n):
     pick = np.sort(np.random.default_rng(3).choice(n, 16, replace=False))
     pick[0], pick[-1] = 0, n - 1
     y1 = oracle.matmul(np.ascontiguousarray(x[pick]), w1, dtype)
-    close(oracle, oracle.matmul(y1, w2, dtype), got[pick], dtype, 1e-2)
+    # The intermediate is rounded to fp16 on both sides, after sums in different orders: single
+    # elements of Y1 differ by an ulp, which is not small relative to the smallest results.  Judged
+    # against the largest result and in rms; a missing barrier gives errors of order one.
+    t, g = (oracle.to_f32(a, dtype).astype(np.float64) for a in (oracle.matmul(y1, w2, dtype), got[pick]))
+    assert np.abs(t - g).max() <= 1e-3 * np.abs(t).max()
+    assert np.sqrt(((t - g) ** 2).mean()) <= 1e-3 * np.sqrt((t * t).mean())
 
 
 def test_iterated_gemm_plus_one_keeps_iteration_barrier(oracle, monkeypatch):
