@@ -197,6 +197,9 @@ int arkmi_model_op(arkmi_model *m, const char *op_c, const int64_t *inputs, int 
         } else if (op == "rope") {
             need_inputs(2);
             res = {M.rope(in(0), in(1), out, name)};
+        } else if (op == "embedding") {
+            need_inputs(2);
+            res = {M.embedding(in(0), in(1), out, name)};
         } else if (op == "swiglu") {
             need_inputs(3);
             res = {M.swiglu(in(0), in(1), in(2), out, name)};

@@ -486,6 +486,36 @@ DevOp lower_op(const Json &op_json, const Lowering &L, int slot_warps, int block
         return d;
     }
 
+    if (type == "Embedding") {
+        View4 in = L.view(op->read_tensors()[0]), w = L.view(op->read_tensors()[1]);
+        View4 out = L.view(op->write_tensors()[0]);
+        if (in.dtype != 3) ARK_ERR(PlanError, "Embedding: the index tensor must be INT32");
+        if (w.dtype != out.dtype || w.dtype < 0 || w.dtype > 2)
+            ARK_ERR(UnsupportedError, "Embedding supports FP32/FP16/BF16 tables and outputs of one type");
+        if (w.shape[0] * w.shape[1] != 1 || w.es[3] != 1 || out.es[3] != 1 || out.shape[3] != w.shape[3])
+            ARK_ERR(PlanError, "Embedding: the table must be [num_embeddings, dim] and the output [..., dim], both dense along dim");
+        EmbedDesc &e = d.emb;
+        e.idx = reinterpret_cast<const int32_t *>(in.ptr);
+        e.weight = w.ptr; e.out = out.ptr;
+        e.rows = out.shape[0] * out.shape[1] * out.shape[2];
+        e.dim_c = (int)out.shape[1]; e.dim_h = (int)out.shape[2];
+        // the indices' [.., a, b, c] line up with the output's [a, b, c, dim]
+        if (in.shape[1] * in.shape[2] * in.shape[3] != e.rows || in.shape[0] != 1)
+            ARK_ERR(PlanError, "Embedding: one index per output row expected");
+        for (int i = 0; i < 3; ++i) {
+            e.idx_s[i] = in.es[i + 1];
+            e.out_s[i] = out.es[i];
+        }
+        e.w_pitch = w.es[2];
+        e.emb_dim = (int)w.shape[3]; e.num_emb = (int)w.shape[2];
+        e.elem = (int)w.elem;
+        if ((int64_t)cfg.at("NumTasks").as_int() * slot_warps < e.rows)
+            ARK_ERR(PlanError, "Embedding: ", cfg.at("NumTasks").as_int(), " tasks of ", slot_warps,
+                    " waves do not cover ", e.rows, " rows");
+        d.kind = DEV_EMBED;
+        return d;
+    }
+
     if (type == "Attention") {
         View4 q = L.view(op->read_tensors()[0]), k = L.view(op->read_tensors()[1]), v = L.view(op->read_tensors()[2]);
         View4 o = L.view(op->write_tensors()[0]);
@@ -1025,7 +1055,8 @@ struct Executor {
                                    ? ((ops[o].gemm.dtype == 0 || ops[o].gemm.trans_a) ? FAM_EXT : FAM_GEMM)
                                : ops[o].kind == DEV_EWISE ? FAM_EWISE
                                : ops[o].kind == DEV_GEMV ? FAM_GEMV
-                               : ops[o].kind == DEV_ATTN ? FAM_ATTN : 0;
+                               : ops[o].kind == DEV_ATTN ? FAM_ATTN
+                               : ops[o].kind == DEV_EMBED ? FAM_EXT : 0;
                 families |= group_fam;
                 h_group_fam.push_back(group_fam);
                 g.trace_offset = (int)trace_len;

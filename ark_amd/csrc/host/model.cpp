@@ -670,6 +670,25 @@ Tensor Model::cast(Tensor input, const DataType &data_type, Tensor output, const
     return ADD_OP(make_unary("Cast", in, output.ref(), data_type.ref()), name);
 }
 
+// embedding (ark/ops/ops_embedding.cpp:10-36): the output takes the indices' shape with the
+// table's row length appended
+Tensor Model::embedding(Tensor input, Tensor weight, Tensor output, const std::string &name) {
+    check_null(input.ref());
+    check_null(weight.ref());
+    auto in = input.ref(), w = weight.ref(), out = output.ref();
+    if (in->shape().ndims() > 3) ARK_ERR(ModelError, "input shape ndims > 3: ", in->shape());
+    if (w->shape().ndims() != 2) ARK_ERR(ModelError, "weight shape ndims != 2: ", w->shape());
+    if (out) {
+        check_same_dtype(w, out);
+    } else {
+        const Dims i4 = in->shape().dims4();
+        out = fresh(w->data_type(), Dims(i4[1], i4[2], i4[3], w->shape()[-1]));
+    }
+    auto op = compute_op("Embedding", {in, w}, out);
+    op->verify();
+    return ADD_OP(op, name);
+}
+
 // transpose (ark/ops/ops_transpose.cpp:37-79)
 Tensor Model::transpose(Tensor input, const std::vector<int64_t> &permutation, Tensor output,
                         const std::string &name) {

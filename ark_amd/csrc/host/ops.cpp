@@ -96,6 +96,14 @@ static Json reference_config(const ModelOp &op, const Arch &arch) {
         // ark/ops/ops_transpose.cpp:110-124
         return tile_config(1, op.result_tensors()[0]->shape().dims4(), 8, 8);
     }
+    if (t == "Embedding") {
+        // ark/ops/ops_embedding.cpp:58-66: one warp per output row
+        Json c = Json::object();
+        c["NumWarps"] = 1; c["SramBytes"] = 0;
+        const Dims s = op.result_tensors()[0]->shape().dims4();
+        c["NumTasks"] = (long long)(s[0] * s[1] * s[2]);
+        return c;
+    }
     if (t == "Noop") {
         Json c = Json::object();
         c["NumWarps"] = 1; c["SramBytes"] = 0; c["NumTasks"] = 0;
@@ -243,6 +251,14 @@ static Json rocm950_config(const ModelOp &op, int num_cu) {
         int64_t tw = std::min<int64_t>(s[3], 4096);
         int64_t th = std::max<int64_t>(1, std::min<int64_t>(s[2], 32768 / tw));
         return tile_config(kWarps950, s, th, tw);
+    }
+    if (t == "Embedding") {
+        // one wave per output row, eight rows per task
+        Json c = Json::object();
+        c["NumWarps"] = kWarps950; c["SramBytes"] = 0;
+        const Dims s = op.result_tensors()[0]->shape().dims4();
+        c["NumTasks"] = (long long)div_up(s[0] * s[1] * s[2], kWarps950);
+        return c;
     }
     if (t == "Noop") {
         Json c = Json::object();

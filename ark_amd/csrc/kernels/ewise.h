@@ -367,6 +367,46 @@ __device__ __forceinline__ void ewise_cast_from(const EwiseDesc &d, int task, co
     }
 }
 
+// ---- embedding gather ---------------------------------------------------------------
+// out[n, c, h, :] = weight[idx[n, c, h], :] with negative indices counted from the end of
+// the table (ark/include/kernels/embedding.h:107-143).  One wave per output row: the
+// index is a uniform load, the row moves as 16-byte vectors when both rows are aligned.
+struct EmbedDesc {
+    const int32_t *idx;
+    const void *weight;
+    void *out;
+    int64_t rows;          // N * C * H of the output
+    int32_t dim_c, dim_h;  // output C and H, to unflatten a row number
+    int64_t idx_s[3];      // element strides of the index tensor along N, C, H
+    int64_t out_s[3];      // element strides of the output rows
+    int64_t w_pitch;       // elements between rows of the table
+    int32_t emb_dim, num_emb;
+    int32_t elem;          // bytes per element (2 or 4)
+    int32_t pad_;
+};
+
+__device__ __forceinline__ void embedding_task(const EmbedDesc &d, int task, const Slot &s) {
+    const int64_t row = (int64_t)task * s.nwaves() + s.wave();
+    if (row >= d.rows) return;
+    const int lane = s.lane();
+    const int64_t h = row % d.dim_h, c = (row / d.dim_h) % d.dim_c, n = row / ((int64_t)d.dim_h * d.dim_c);
+    int e = as_global(d.idx)[n * d.idx_s[0] + c * d.idx_s[1] + h * d.idx_s[2]];
+    if (e < 0) e += d.num_emb;
+    e = __builtin_amdgcn_readfirstlane(e);
+    gptr<const char> src = as_global(static_cast<const char *>(d.weight)) + (int64_t)e * d.w_pitch * d.elem;
+    gptr<char> dst = as_global(static_cast<char *>(d.out)) +
+                     (n * d.out_s[0] + c * d.out_s[1] + h * d.out_s[2]) * d.elem;
+    const int bytes = d.emb_dim * d.elem;
+    if ((((uintptr_t)src | (uintptr_t)dst | (uintptr_t)bytes) & 15) == 0) {
+        for (int b = lane * 16; b < bytes; b += 64 * 16)
+            store16<char>(dst + b, load16<char>(src + b));
+    } else if (d.elem == 4) {
+        for (int i = lane; i < d.emb_dim; i += 64) ((gptr<uint32_t>)dst)[i] = ((gptr<const uint32_t>)src)[i];
+    } else {
+        for (int i = lane; i < d.emb_dim; i += 64) ((gptr<uint16_t>)dst)[i] = ((gptr<const uint16_t>)src)[i];
+    }
+}
+
 __device__ __forceinline__ void ewise_dispatch(const EwiseDesc &d, int task, const Slot &s) {
     if (d.op == EW_CAST || d.dt_in != d.dt_out) {
         switch (d.dt_in) {

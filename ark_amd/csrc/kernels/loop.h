@@ -21,12 +21,12 @@
 
 namespace arkmi {
 
-enum DevOpKind : int32_t { DEV_NOOP = 0, DEV_ROW = 1, DEV_GEMM = 2, DEV_EWISE = 3, DEV_GEMV = 4, DEV_ATTN = 5 };
+enum DevOpKind : int32_t { DEV_NOOP = 0, DEV_ROW = 1, DEV_GEMM = 2, DEV_EWISE = 3, DEV_GEMV = 4, DEV_ATTN = 5, DEV_EMBED = 6 };
 
 // Op families as a bit set: which bodies a loop-kernel variant carries, and
 // which a compiled plan needs.
 // FAM_EXT holds the bodies few plans use (fp32 and transposed-first-operand matmuls,
-// reductions over an axis other than the last): kept out of the common variants, whose
+// reductions over an axis other than the last, the embedding gather): kept out of the common variants, whose
 // register allocation and code size every other body shares.
 enum OpFamily : int32_t { FAM_ROW = 1, FAM_EWISE = 2, FAM_GEMM = 4, FAM_GEMV = 8, FAM_ATTN = 16, FAM_EXT = 32,
                           FAM_ALL = 63 };
@@ -41,6 +41,7 @@ struct DevOp {
         GemvDesc gemv;
         AttnDesc attn;
         EwiseDesc ew;
+        EmbedDesc emb;
     };
 };
 

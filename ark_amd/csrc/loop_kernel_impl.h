@@ -244,6 +244,12 @@ __device__ __forceinline__ void run_op(const DevOp *op, int task, const Slot &s_
                 gemv_dispatch(d, task, s);
             }
             break;
+        case DEV_EMBED:
+            if constexpr ((FAM & FAM_EXT) != 0) {
+                const EmbedDesc d = load_const(&op->emb);
+                embedding_task(d, task, s);
+            }
+            break;
         case DEV_ATTN:
             if constexpr ((FAM & FAM_ATTN) != 0) {
                 const AttnDesc d = load_const(&op->attn);

@@ -233,6 +233,9 @@ class Model:
     def rope(self, input, other, output=None, name=""):
         return self._op1("rope", [input, other], output, name)
 
+    def embedding(self, input, weight, output=None, name=""):
+        return self._op1("embedding", [input, weight], output, name)
+
     def transpose(self, input, permutation, output=None, name=""):
         return self._op1("transpose", [input], output, name, permutation=list(permutation))
 

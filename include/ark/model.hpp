@@ -114,6 +114,9 @@ class Model : public ModelGraph {
     Tensor silu_mul(Tensor input, Tensor other, Tensor output = NullTensor, const std::string &name = "");
     Tensor rope(Tensor input, Tensor other, Tensor output = NullTensor,
                 const std::string &name = "");
+    // Rows of `weight` [num_embeddings, dim] picked by the INT32 indices of `input` (at
+    // most 3-D); negative indices count from the end of the table.
+    Tensor embedding(Tensor input, Tensor weight, Tensor output = NullTensor, const std::string &name = "");
     // 4-D permutation copy.
     Tensor transpose(Tensor input, const std::vector<int64_t> &permutation,
                      Tensor output = NullTensor, const std::string &name = "");

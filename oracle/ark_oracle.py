@@ -247,6 +247,15 @@ def cast(x, src, dst):
     return out
 
 
+def embedding(indices, weight):
+    """out[..., :] = weight[indices[...], :], negative indices counted from the end of the
+    table (the host baseline of ark/ops/ops_embedding_test.cpp:11-41).  Pure data movement:
+    works on the storage bits of any type."""
+    idx = np.asarray(indices, dtype=np.int64)
+    idx = np.where(idx < 0, idx + weight.shape[0], idx)
+    return np.ascontiguousarray(weight[idx])
+
+
 def tensor_compare(truth, got, dtype):
     """Returns dict(mse, max_diff, max_error_rate, num_wrong, num_total)."""
     truth = _c(truth, dtype)

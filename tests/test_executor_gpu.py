@@ -754,3 +754,101 @@ def test_elided_barriers_give_the_reference_placements_results(oracle, graph, mo
         outs.append(got)
     for a, b in zip(*outs):
         assert np.array_equal(a, b), graph
+
+
+# ---------------------------------------------------------------- remaining single-GPU ops
+@pytest.mark.parametrize("dtype", ["fp32", "fp16", "bf16"])
+def test_embedding(oracle, dtype):
+    """ops_embedding_test.cpp:43-96: indices [8, 3, 64] into a [100, 4096] table, every ninth index
+    negative (counted from the end of the table); exact."""
+    from ark_amd import Model
+    num_emb, dim = 100, 4096
+    rng = np.random.default_rng(12)
+    idx = rng.integers(0, num_emb, (8, 3, 64)).astype(np.int32)
+    flat = idx.reshape(-1)
+    flat[::9] = -flat[::9]
+    w = make(oracle, (num_emb, dim), dtype, 13, "uniform")
+    m = Model()
+    ti, tw = m.tensor(idx.shape, "int32"), m.tensor(w.shape, dtype)
+    out = m.embedding(ti, tw)
+    assert out.shape == [8, 3, 64, dim]
+    (got,), ex, _ = run_model(m, {ti: idx, tw: w}, [out], iters=2)
+    assert np.array_equal(got, oracle.embedding(idx, w))
+
+
+def test_embedding_ragged_rows_and_other_ops_in_one_plan(oracle):
+    """A table whose rows are not whole 16-byte vectors (scalar path), a 1-D index vector, and a
+    matmul on the gathered rows in the same plan."""
+    from ark_amd import Model
+    dtype = "fp16"
+    idx = np.array([3, -1, 0, 7, -8, 5, 5, 2, 1], np.int32)
+    w = make(oracle, (8, 50), dtype, 14, "uniform")
+    w2 = make(oracle, (16, 128), dtype, 15, "uniform")
+    b = make(oracle, (128, 128), dtype, 16, "uniform")
+    idx2 = np.arange(-128, 0, dtype=np.int32).reshape(128) % 16 - 16  # all negative
+    m = Model()
+    ti, tw = m.tensor(idx.shape, "int32"), m.tensor(w.shape, dtype)
+    ti2, tw2, tb = m.tensor(idx2.shape, "int32"), m.tensor(w2.shape, dtype), m.tensor(b.shape, dtype)
+    o1 = m.embedding(ti, tw)
+    g2 = m.embedding(ti2, tw2)
+    assert o1.shape == [1, 1, 9, 50] and g2.shape == [1, 1, 128, 128]
+    o2 = m.matmul(m.reshape(g2, [128, 128]), tb)
+    (got1, got2), _, _ = run_model(m, {ti: idx, tw: w, ti2: idx2, tw2: w2, tb: b}, [o1, o2])
+    assert np.array_equal(got1.reshape(9, 50), oracle.embedding(idx, w))
+    close(oracle, oracle.matmul(oracle.embedding(idx2, w2), b, dtype), got2, dtype, 1e-2)
+
+
+def _all_permutations():
+    import itertools
+    return [p for p in itertools.permutations(range(4)) if p != (0, 1, 2, 3)]
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16", "bf16"])
+def test_transpose_all_permutations(oracle, dtype):
+    """All 23 non-identity permutations of a 4-D tensor (the reference instantiates one kernel per
+    permutation, ark/include/kernels/transpose.h, and tests 0132 and 0231 in three types,
+    ops_transpose_test.cpp:154-160); one plan per type holds all of them.  Exact."""
+    from ark_amd import Model
+    x = make(oracle, (3, 4, 24, 40), dtype, 18)
+    m = Model()
+    t = m.tensor(x.shape, dtype)
+    outs = [m.transpose(t, list(p)) for p in _all_permutations()]
+    got, _, _ = run_model(m, {t: x}, outs)
+    for p, g in zip(_all_permutations(), got):
+        assert np.array_equal(g, np.transpose(x, p)), p
+    # the two shapes the reference tests: [5, 3, 32, 128] as 0132 and 0231
+    y = make(oracle, (5, 3, 32, 128), dtype, 19)
+    m = Model()
+    t = m.tensor(y.shape, dtype)
+    outs = [m.transpose(t, [0, 1, 3, 2]), m.transpose(t, [0, 2, 3, 1])]
+    got, _, _ = run_model(m, {t: y}, outs)
+    assert np.array_equal(got[0], np.transpose(y, (0, 1, 3, 2)))
+    assert np.array_equal(got[1], np.transpose(y, (0, 2, 3, 1)))
+
+
+@pytest.mark.parametrize("dtype", ["fp32", "fp16", "int32"])
+def test_cast_through_bytes(oracle, dtype):
+    """Casts to and from BYTE reinterpret the buffer (ops_cast_test.cpp:141-233, ops_cast.cpp:107-132):
+    a tensor seen as bytes, a byte tensor seen as `dtype`, and a real op on the reinterpreted view so
+    that the plan reads it on the GPU."""
+    from ark_amd import Model
+    elem = 2 if dtype == "fp16" else 4
+    rng = np.random.default_rng(20)
+    raw = rng.integers(0, 256, (4, 2, 1024), dtype=np.uint8)
+    if dtype != "int32":
+        # keep the reinterpreted floats finite: clear the top exponent bit of every element
+        raw.reshape(-1, elem)[:, elem - 1] &= 0xBF
+    m = Model()
+    tb = m.tensor(raw.shape, "byte")
+    as_t = m.cast(tb, dtype)            # view: [4, 2, 1024 / elem]
+    assert as_t.shape == [4, 2, 1024 // elem] and as_t.buffer_id == tb.buffer_id
+    back = m.cast(as_t, "byte")         # and back: the original bytes
+    assert back.shape == list(raw.shape) and back.buffer_id == tb.buffer_id
+    copied = m.copy(as_t)               # a kernel that reads the reinterpreted view
+    m.noop(back)
+    (g_t, g_back, g_copy), _, _ = run_model(m, {tb: raw}, [as_t, back, copied])
+    np_t = {"fp32": np.float32, "fp16": np.float16, "int32": np.int32}[dtype]
+    want = raw.view(np_t)
+    assert np.array_equal(g_t.view(np.uint8), raw) and g_t.shape == want.shape
+    assert np.array_equal(g_back, raw)
+    assert np.array_equal(g_copy.view(np.uint8).reshape(raw.shape), raw)

@@ -324,3 +324,24 @@ def test_fused_op_plans_exist_only_on_rocm950():
     with pytest.raises(ArkmiError) as e:
         m.plan(arch="CUDA_80", num_processors=108)
     assert e.value.kind == "PlanError"
+
+
+def test_embedding_shapes_and_invalid():
+    """ops_embedding.cpp:10-36, ops_embedding_test.cpp:98-112."""
+    m = Model()
+    ti = m.tensor([8, 3, 64], "int32")
+    tw = m.tensor([100, 4096], "fp16")
+    out = m.embedding(ti, tw)
+    assert out.shape == [8, 3, 64, 4096] and out.dtype == "fp16"
+    assert m.embedding(m.tensor([7], "int32"), tw).shape == [1, 1, 7, 4096]
+    raises_model_error(lambda: m.embedding(m.tensor([4, 8, 3, 64], "int32"), m.tensor([100, 1024], "fp32")))
+    raises_model_error(lambda: m.embedding(ti, m.tensor([2, 100, 1024], "fp32")))
+    raises_model_error(lambda: m.embedding(ti, tw, m.tensor([8, 3, 64, 4096], "fp32")))  # output type != table type
+    # default configs: one warp per row on the reference's architectures, one wave per row here
+    import json
+    p = json.loads(m.plan(arch="CUDA_80", num_processors=108))
+    cfg = p["TaskInfos"][0]["Ops"][0]["Config"]
+    assert cfg["NumWarps"] == 1 and cfg["NumTasks"] == 8 * 3 * 64
+    p = json.loads(m.plan(arch="ROCM_950", num_processors=256))
+    cfg = p["TaskInfos"][0]["Ops"][0]["Config"]
+    assert cfg["NumWarps"] == 8 and cfg["NumTasks"] == 8 * 3 * 64 // 8
