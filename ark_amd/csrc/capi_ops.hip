@@ -185,7 +185,7 @@ extern "C" int arkmi_gemm(int dtype, const void *a, const void *b, void *c, int 
         d.lda = (int)lda; d.ldb = (int)ldb; d.ldc = (int)ldc;
         d.a_bs[0] = d.b_bs[0] = d.c_bs[0] = 0;
         d.a_bs[1] = batch_stride_a; d.b_bs[1] = batch_stride_b; d.c_bs[1] = batch_stride_c;
-        d.batch_c = batch; d.trans_b = trans_b; d.trans_a = trans_a ? 1 : 0; d.dtype = dtype;
+        d.batch_c = batch; d.batch_total = batch; d.split_k = 1; d.trans_b = trans_b; d.trans_a = trans_a ? 1 : 0; d.dtype = dtype;
         d.tiles_m = m / tile_m; d.tiles_n = n / tile_n;
         d.store_m = m; d.store_n = n;
         int64_t ntasks = (int64_t)batch * d.tiles_m * d.tiles_n;

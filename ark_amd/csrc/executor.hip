@@ -313,6 +313,8 @@ DevOp lower_op(const Json &op_json, const Lowering &L, int slot_warps, int block
         }
         g.trans_b = 1;
         g.dtype = a.dtype;
+        g.split_k = 1;
+        g.batch_total = (int)(c.shape[0] * c.shape[1]);
         g.tiles_m = (int)(M / tm); g.tiles_n = (int)(H / 128);
         g.store_m = (int)M; g.store_n = (int)H;
         if ((int64_t)cfg.at("NumTasks").as_int() != c.shape[0] * c.shape[1] * g.tiles_m * g.tiles_n)
@@ -397,6 +399,24 @@ DevOp lower_op(const Json &op_json, const Lowering &L, int slot_warps, int block
         g.dtype = a.dtype;
         g.tiles_m = g.m / tm; g.tiles_n = g.n / tn;
         g.store_m = (int)c.shape[2]; g.store_n = (int)c.shape[3];
+        g.batch_total = (int)(c.shape[0] * c.shape[1]);
+        g.split_k = cfg.contains("SplitK") ? (int)cfg.at("SplitK").as_int() : 1;
+        const int64_t tiles = (int64_t)g.batch_total * g.tiles_m * g.tiles_n;
+        if (g.split_k != 1 && g.split_k != 2) ARK_ERR(PlanError, "Matmul: SplitK must be 1 or 2, got ", g.split_k);
+        if ((int64_t)cfg.at("NumTasks").as_int() != tiles * g.split_k)
+            ARK_ERR(PlanError, "Matmul: NumTasks must be SplitK * batch * (M / ", tm, ") * (N / ", tn, ") = ",
+                    tiles * g.split_k, ", got ", cfg.at("NumTasks").as_int());
+        if (g.split_k == 2) {
+            if (tm != 256 || tn != 256 || ta || f32 || (g.k % (4 * kGemmMinK / 2)))
+                ARK_ERR(UnsupportedError, "Matmul: SplitK 2 runs on 256x256 tiles of FP16/BF16 operands with K % ",
+                        2 * kGemmMinK, " == 0 and no TransposeInput");
+            // partial accumulators of both halves + one arrival counter per tile
+            const size_t counter_bytes = ((size_t)tiles * 4 + 255) / 256 * 256;
+            const size_t tile_bytes = (size_t)2 * kGemmThreads * (256 / 2 / 16) * (256 / 4 / 16) * 16;
+            char *ws = static_cast<char *>(L.scratch(counter_bytes + (size_t)tiles * tile_bytes));
+            g.arrivals = reinterpret_cast<unsigned int *>(ws);
+            g.partial = reinterpret_cast<float *>(ws + counter_bytes);
+        }
         d.kind = DEV_GEMM;
         d.gemm_tile_m = tm; d.gemm_tile_n = tn;
         return d;
@@ -690,7 +710,8 @@ struct Access {
 
 bool tiled_elementwise(const std::string &type);
 
-void add_access(std::vector<Access> &out, const Json &tensor_json, bool write, const std::string &op_type) {
+void add_access(std::vector<Access> &out, const Json &tensor_json, bool write, const std::string &op_type,
+                bool split_k) {
     auto t = ark::ModelTensor::deserialize(tensor_json);
     ark::Dims st = t->strides(), pd = t->padded_shape();
     size_t last = 0, pitch = 1;
@@ -700,7 +721,8 @@ void add_access(std::vector<Access> &out, const Json &tensor_json, bool write, c
     }
     const size_t elem = t->data_type()->bytes();
     Access a{t->buffer()->id(), t->byte_offset(), t->byte_offset() + (last + 1) * elem, write, "", t->shape(), -1};
-    a.tile_local = tiled_elementwise(op_type) || (write && op_type == "Matmul");
+    // (a matmul that splits K is finished by whichever half arrives last: no fixed workgroup)
+    a.tile_local = tiled_elementwise(op_type) || (write && op_type == "Matmul" && !split_k);
     a.panel_read = !write && (op_type == "Matmul" || op_type == "MatmulSwiglu" || op_type == "Attention");
     a.view = tensor_json.at("DataType").dump() + tensor_json.at("Shape").dump() + tensor_json.at("Strides").dump() +
              tensor_json.at("Offsets").dump() + tensor_json.at("PaddedShape").dump();
@@ -711,9 +733,11 @@ std::vector<Access> accesses_of(const Json &task_info) {
     std::vector<Access> v;
     for (const auto &op : task_info.at("Ops").elements()) {
         const std::string type = op.at("Type").as_string();
-        for (const auto &t : op.at("ReadTensors").elements()) add_access(v, t, false, type);
-        for (const auto &t : op.at("WriteTensors").elements()) add_access(v, t, true, type);
-        for (const auto &t : op.at("ResultTensors").elements()) add_access(v, t, true, type);
+        const Json &cfg = op.at("Config");
+        const bool split = cfg.contains("SplitK") && cfg.at("SplitK").as_int() > 1;
+        for (const auto &t : op.at("ReadTensors").elements()) add_access(v, t, false, type, split);
+        for (const auto &t : op.at("WriteTensors").elements()) add_access(v, t, true, type, split);
+        for (const auto &t : op.at("ResultTensors").elements()) add_access(v, t, true, type, split);
     }
     return v;
 }
@@ -758,6 +782,7 @@ Tiling tiling_of(const Json &task_info) {
             auto tile = cfg.at("TileShapeMNK").as_int_vector();
             th = tile.at(0); tw = tile.at(1);
             if (th < 32) return Tiling();  // the skinny matmul deals units of W, not output tiles
+            if (cfg.contains("SplitK") && cfg.at("SplitK").as_int() > 1) return Tiling();  // no fixed workgroup per tile
         } else if (tiled_elementwise(type) && cfg.contains("Tile")) {
             auto tile = cfg.at("Tile").as_int_vector();
             th = tile.at(0); tw = tile.at(1);
@@ -1038,8 +1063,10 @@ struct Executor {
                 // (an op with no tasks, such as Noop, aside)
                 int64_t common_tasks = -1;
                 for (const auto &oj : ops_json.elements()) {
-                    const int64_t nt = oj.at("Config").at("NumTasks").as_int();
+                    int64_t nt = oj.at("Config").at("NumTasks").as_int();
                     if (nt == 0) continue;
+                    // a matmul that splits K runs SplitK tasks per tile; its followers one per tile
+                    if (oj.at("Config").contains("SplitK")) nt /= std::max<int64_t>(1, oj.at("Config").at("SplitK").as_int());
                     if (common_tasks < 0) common_tasks = nt;
                     if (nt != common_tasks)
                         ARK_ERR(PlanError, "the ops fused into task ", st.task_info, " have different NumTasks (", common_tasks,
@@ -1052,7 +1079,8 @@ struct Executor {
                 for (int o = g.op_begin; o < (int)ops.size(); ++o)
                     group_fam |= ops[o].kind == DEV_ROW ? (ops[o].row.red_len > 0 ? FAM_EXT : FAM_ROW)
                                : ops[o].kind == DEV_GEMM
-                                   ? ((ops[o].gemm.dtype == 0 || ops[o].gemm.trans_a) ? FAM_EXT : FAM_GEMM)
+                                   ? ((ops[o].gemm.dtype == 0 || ops[o].gemm.trans_a) ? FAM_EXT
+                                      : ops[o].gemm.split_k == 2 ? (FAM_GEMM | FAM_SPLITK) : FAM_GEMM)
                                : ops[o].kind == DEV_EWISE ? FAM_EWISE
                                : ops[o].kind == DEV_GEMV ? FAM_GEMV
                                : ops[o].kind == DEV_ATTN ? FAM_ATTN
@@ -1094,7 +1122,7 @@ struct Executor {
             if (whole_grid_only) {
                 auto has_scratch = [&](int sj) {
                     const DevStep &dst = steps[(size_t)dev_step_of[(size_t)sj]];
-                    return (h_group_fam[(size_t)dst.index] & FAM_GEMV) != 0;
+                    return (h_group_fam[(size_t)dst.index] & (FAM_GEMV | FAM_SPLITK)) != 0;
                 };
                 std::vector<Access> tail, head;
                 for (size_t sj = (size_t)(last_full + 1); sj < sched.steps.size(); ++sj)

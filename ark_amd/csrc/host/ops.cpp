@@ -167,13 +167,25 @@ static Json rocm950_config(const ModelOp &op, int num_cu) {
         if (tm == 0 || mnk[2] % 64 != 0)
             ARK_ERR(PlanError, "output padded shape MNK ", mnk,
                     " should be divisible by a tile shape of 128x128x64 or larger");
+        // An output that gives 256x256 tiles to between half and all of the CUs: keep the large
+        // tile (half the operand traffic per flop of a 128x256 tile) and split K in two, so the
+        // tiles' halves fill the chip; the half that finishes second adds the two.
+        int64_t split = 1;
+        if (!trans_in && !f32 && mnk[0] % 256 == 0 && mnk[1] % 256 == 0 && mnk[2] % 128 == 0 && mnk[2] >= 2048) {
+            const int64_t tiles256 = batch * (mnk[0] / 256) * (mnk[1] / 256);
+            if (tiles256 < num_cu && 2 * tiles256 >= num_cu) {
+                tm = tn = 256;
+                split = 2;
+            }
+        }
         Json c = Json::object();
         c["NumWarps"] = kWarps950;
         c["SramBytes"] = gemm_lds_bytes((int)tm, (int)tn);
         Json tile = Json::array();
         tile.push_back((long long)tm); tile.push_back((long long)tn); tile.push_back(64);
         c["TileShapeMNK"] = tile;
-        c["NumTasks"] = (long long)(batch * (mnk[0] / tm) * (mnk[1] / tn));
+        if (split > 1) c["SplitK"] = (long long)split;
+        c["NumTasks"] = (long long)(split * batch * (mnk[0] / tm) * (mnk[1] / tn));
         return c;
     }
     if (t == "MatmulSwiglu") {

@@ -51,20 +51,7 @@ constexpr int kAttnVPitch = kAttnD * 2 + 32;  // LDS row pitch of the V tile (by
 constexpr int kAttnStageBytes = kAttnKBlock * (kAttnKPitch + kAttnVPitch);
 constexpr int kAttnLdsBytes = 2 * kAttnStageBytes;
 
-typedef float f32x4v __attribute__((ext_vector_type(4)));
-
-template <typename T>
-__device__ __forceinline__ f32x4v mfma16x32(u32x4 a, u32x4 b, f32x4v c);
-template <>
-__device__ __forceinline__ f32x4v mfma16x32<f16>(u32x4 a, u32x4 b, f32x4v c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
-                                                  0);
-}
-template <>
-__device__ __forceinline__ f32x4v mfma16x32<bf16>(u32x4 a, u32x4 b, f32x4v c) {
-    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
-                                                   0, 0);
-}
+using f32x4v = f32x4;  // the 16x16x32 MFMA wrappers live in gemm.h
 
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {

@@ -4,12 +4,27 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+#include <utility>
+
 namespace arkmi {
 
 using f16 = _Float16;
 using bf16 = __bf16;
 
 constexpr int kWave = 64;
+
+// ---- compile-time loops ---------------------------------------------------------
+// static_for<N>(f) calls f(std::integral_constant<int, I>{}) for I = 0 .. N-1: for bodies whose
+// instructions need the index as a constant (scheduling hints, register-array slots).
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F &&f) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
 
 // ---- storage <-> float ----------------------------------------------------
 template <typename T>

@@ -2,7 +2,9 @@
 // accumulate, one rounding to the storage type.
 //
 // One task = one BM x BN output tile, computed by the 8 waves of a workgroup
-// (2 x 4 wave grid) with v_mfma_f32_32x32x16.  A and B tiles of depth BK
+// (2 x 4 wave grid) with v_mfma_f32_16x16x32 (at the chip's power limit that shape
+// sustains about 15 % more flops than 32x32x16: a quarter of the accumulator
+// traffic per instruction for half the flops).  A and B tiles of depth BK
 // travel from global memory straight into LDS (global_load_lds_dwordx4, no
 // staging registers, no LDS store instructions) into a ring of S stage
 // buffers; the loads of the next S-1 tiles are in flight while the current one
@@ -39,6 +41,7 @@ struct GemmDesc {
     // batch_c, c = idx % batch_c; a stride of 0 broadcasts the operand.
     int64_t a_bs[2], b_bs[2], c_bs[2];
     int32_t batch_c;
+    int32_t batch_total;       // number of (N, C) batches
     int32_t trans_b;           // 1: B stored [N,K]; 0: B stored [K,N]
     int32_t trans_a;           // 1: A stored [K,M] (128x128 tiles only); 0: A stored [M,K]
     // Gate/up pair (b2 != null, trans_b): C[M, n/2] = silu(A . B^T) * (A . B2^T) with B, B2 stored
@@ -48,6 +51,13 @@ struct GemmDesc {
     int32_t dtype;             // 1 fp16, 2 bf16; 0 fp32 (kernels/gemm_f32.h, 128x128 tiles)
     int32_t tiles_m, tiles_n;  // ceil(m/BM), ceil(n/BN)
     int32_t store_m, store_n;  // rows/cols of C that exist (unpadded shape)
+    // Two-way split of K (split_k == 2): task t and task t + tiles each multiply half of K for
+    // tile t; both leave their fp32 accumulators in `partial` and count in `arrivals[t]`; the one
+    // that arrives second adds the other's and finishes the tile.  Nobody waits.
+    int32_t split_k;           // 1 or 2
+    int32_t pad_;
+    float *partial;            // [tiles][2][512 threads][MT * NT] x 4 floats
+    unsigned int *arrivals;    // [tiles], zero between uses
 };
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -59,18 +69,20 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 using lds_u32x4 = __attribute__((address_space(3))) u32x4;
 using lds_s16x4 = __attribute__((address_space(3))) s16x4;
 using lds_void = __attribute__((address_space(3))) void;
+using lds_i32x = __attribute__((address_space(3))) int;
 
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 template <typename T>
-__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c);
+__device__ __forceinline__ f32x4 mfma16x32(u32x4 a, u32x4 b, f32x4 c);
 template <>
-__device__ __forceinline__ f32x16 mfma32<f16>(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+__device__ __forceinline__ f32x4 mfma16x32<f16>(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0,
+                                                  0);
 }
 template <>
-__device__ __forceinline__ f32x16 mfma32<bf16>(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+__device__ __forceinline__ f32x4 mfma16x32<bf16>(u32x4 a, u32x4 b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0,
+                                                   0, 0);
 }
 
 constexpr int kGemmThreads = 512;
@@ -112,16 +124,29 @@ struct EpilogueStore {
     __device__ __forceinline__ float operator()(float v, int, int) const { return v; }
 };
 
-template <typename T, int BM, int BN, bool TRANS_B, typename Epi, bool TRANS_A = false, bool DUAL_B = false>
-__device__ __forceinline__ void gemm_tile(const GemmDesc &d, int task, const Slot &s, Epi epi) {
+// Returns the tile this workgroup finished (its followers — the elementwise ops fused behind the
+// matmul — run for that tile index), or -1 when the other half of a split tile will finish it.
+template <typename T, int BM, int BN, bool TRANS_B, typename Epi, bool TRANS_A = false, bool DUAL_B = false,
+          bool SPLIT = false>
+__device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const Slot &s, Epi epi) {
     static_assert(!DUAL_B || (TRANS_B && !TRANS_A), "the gate/up pair takes K-contiguous operands");
+    static_assert(!SPLIT || (!DUAL_B && !TRANS_A), "the split of K exists for plain matmuls");
+    // split: tasks [0, tiles) take the upper half of K, tasks [tiles, 2 tiles) the lower half
+    int task = task_in, k_begin = 0, k_len = d.k, half = 0;
+    if constexpr (SPLIT) {
+        const int tiles = d.tiles_m * d.tiles_n * d.batch_total;
+        half = task_in >= tiles ? 0 : 1;
+        task = task_in >= tiles ? task_in - tiles : task_in;
+        k_len = d.k / 2;
+        k_begin = half * k_len;
+    }
     constexpr int BK = GemmShape<BM, BN>::BK;
     constexpr int S = GemmShape<BM, BN>::STAGES;
     constexpr int WGM = 2, WGN = 4;                // wave grid
     constexpr int WTM = BM / WGM, WTN = BN / WGN;  // wave tile
-    constexpr int MT = WTM / 32, NT = WTN / 32;    // 32x32 MFMA tiles per wave
+    constexpr int MT = WTM / 16, NT = WTN / 16;    // 16x16 MFMA tiles per wave
     static_assert(MT >= 1 && NT >= 1, "tile too small for the wave grid");
-    static_assert(BK == 16 || BK == 32 || BK == 64, "K tile depth");
+    static_assert(BK == 32 || BK == 64, "K tile depth");
     using L = GemmLds<BM, BN>;
     constexpr int ROW_B = 2 * BK;                    // bytes per row of a K-contiguous tile
     constexpr int CPR_K = BK / 8;                    // 16-byte chunks per such row
@@ -153,8 +178,10 @@ __device__ __forceinline__ void gemm_tile(const GemmDesc &d, int task, const Slo
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int bn = bidx / d.batch_c, bc = bidx % d.batch_c;
-    gptr<const T> A = as_global(static_cast<const T *>(d.a) + bn * d.a_bs[0] + bc * d.a_bs[1]);
-    gptr<const T> B = as_global(static_cast<const T *>(d.b) + bn * d.b_bs[0] + bc * d.b_bs[1]);
+    // k_begin moves both operands along K (only the plain layouts can be split)
+    gptr<const T> A = as_global(static_cast<const T *>(d.a) + bn * d.a_bs[0] + bc * d.a_bs[1] + k_begin);
+    gptr<const T> B = as_global(static_cast<const T *>(d.b) + bn * d.b_bs[0] + bc * d.b_bs[1] +
+                                (TRANS_B ? (int64_t)k_begin : (int64_t)k_begin * d.ldb));
     gptr<T> C = as_global(static_cast<T *>(d.c) + bn * d.c_bs[0] + bc * d.c_bs[1]);
 
     const lds_ptr lds = s.lds;
@@ -231,87 +258,90 @@ __device__ __forceinline__ void gemm_tile(const GemmDesc &d, int task, const Slo
     };
 
     // ---- LDS fragment addresses -------------------------------------------------------
-    // A operand of mfma 32x32x16: lane holds row (lane%32), k = (lane/32)*8..+7, that
-    // is k-group 2*kk + lane/32 of its row.  Wave and MFMA tile offsets are
-    // multiples of 32 rows, so the swizzle depends on the lane alone.
-    const int l32 = lane & 31;
-    const int sw = (BK == 64) ? ((l32 & 7) ^ ((l32 >> 3) & 1)) : (BK == 32) ? ((l32 >> 2) & 3) : ((l32 >> 3) & 1);
-    int kx[BK / 16];
+    // v_mfma_f32_16x16x32 takes, per lane, 8 consecutive k of one row (first operand) or one
+    // column (second operand): lane -> row/column lane%16, k-group lane/16.  The operands are
+    // swapped — the B fragment goes in first, the A fragment second — so the accumulator tile is
+    // C^T: lane (lane%16 = m, lane/16 = g) holds C[m][4g .. 4g+3] of its 16x16 tile, four
+    // consecutive columns, which leave as one 8-byte store.
+    // K-contiguous tiles: the fragment of 16 consecutive rows at one k-group; wave and MFMA tile
+    // offsets are multiples of 16 rows, so the swizzle depends on the lane alone.
+    const int l16 = lane & 15, g4 = lane >> 4;
+    const int sw = (BK == 64) ? ((l16 & 7) ^ ((l16 >> 3) & 1)) : (BK == 32) ? ((l16 >> 2) & 3) : 0;
+    constexpr int KS = BK / 32;  // MFMA k-steps per K tile
+    int kx[KS];
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) kx[kk] = ((kk * 2 + (lane >> 5)) ^ sw) << 4;
-    const int a_frag = (wm * WTM + l32) * ROW_B;
-    const int bt_frag = L::A_BYTES + (wn * WTN + l32) * ROW_B;
-    // B operand, [k][n] layout through ds_read_b64_tr_b16: inside each block of
-    // 16 lanes, lane i supplies the address of 4 consecutive n at k-row (i/4)
-    // and receives 4 consecutive k for column i.  Blocks 0/1 cover n 0-15 /
-    // 16-31 for k 0-7, blocks 2/3 the same columns for k 8-15.
-    const int i16 = lane & 15;
+    for (int ks = 0; ks < KS; ++ks) kx[ks] = ((ks * 4 + g4) ^ sw) << 4;
+    const int a_frag = (wm * WTM + l16) * ROW_B;
+    const int bt_frag = L::A_BYTES + (wn * WTN + l16) * ROW_B;
+    // N-contiguous B tile ([k][n]) through ds_read_b64_tr_b16: inside each block of 16 lanes,
+    // lane i supplies the address of 4 consecutive n at k-row (i/4) and receives 4 consecutive
+    // k for column i.  Block g covers k-rows 8g .. 8g+7 of the k-step in two reads (rows 0-3
+    // and 4-7 of its group), all four blocks the same 16 columns.
     int bn_frag[NT];
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-        const int nchunk = (wn * WTN + j * 32) / 8 + ((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1);
-        bn_frag[j] = L::A_BYTES + ((lane >> 5) * 8 + (i16 >> 2)) * RB_N +
-                     ((nchunk ^ (((i16 >> 2) & 3) << 2)) << 4) + (i16 & 1) * 8;
+        const int nchunk = (wn * WTN + j * 16) / 8 + ((l16 & 3) >> 1);
+        bn_frag[j] = L::A_BYTES + (g4 * 8 + (l16 >> 2)) * RB_N + ((nchunk ^ (((l16 >> 2) & 3) << 2)) << 4) +
+                     (l16 & 1) * 8;
     }
-
     // A operand from an M-contiguous tile ([k][m]): the same transposing reads, m for n
     int am_frag[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
-        const int mchunk = (wm * WTM + i * 32) / 8 + ((lane >> 4) & 1) * 2 + ((i16 & 3) >> 1);
-        am_frag[i] = ((lane >> 5) * 8 + (i16 >> 2)) * RB_M + ((mchunk ^ (((i16 >> 2) & 3) << 2)) << 4) + (i16 & 1) * 8;
+        const int mchunk = (wm * WTM + i * 16) / 8 + ((l16 & 3) >> 1);
+        am_frag[i] = (g4 * 8 + (l16 >> 2)) * RB_M + ((mchunk ^ (((l16 >> 2) & 3) << 2)) << 4) + (l16 & 1) * 8;
     }
 
-    f32x16 acc[MT][NT];
+    f32x4 acc[MT][NT];
 #pragma unroll
     for (int i = 0; i < MT; ++i)
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+        for (int j = 0; j < NT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // ---- main loop -----------------------------------------------------------------
-    // At the top of tile kt one barrier establishes two facts: tile kt+1 has landed
-    // for every wave (each waited for its own loads first), and every wave is
-    // done reading tile kt-1, whose stage is refilled right away.  Because tile
-    // kt+1 is already complete, the fragments of its first k-step are read
-    // during the last k-step of tile kt: the MFMA queue stays fed across the
-    // barrier.  Tiles kt+2 .. kt+S-1 are in flight meanwhile.  A tile index
-    // past the last one is clamped: the extra loads land in a stage nobody
-    // reads again and keep the number of outstanding loads the same in every
-    // iteration, so one constant vmcnt bound serves the whole loop.
-    static_assert(S >= 3, "the ring needs the current, the next and one tile in flight");
-    constexpr int KK = BK / 16;
-    const int KT = d.k / BK;
-    auto read_frags = [&](int stage, int kk, u32x4(&af)[MT], u32x4(&bf)[NT]) {
+    auto read_a = [&](int stage, int ks, int i) -> u32x4 {
         const lds_ptr base = lds + stage * L::STAGE_BYTES;
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            if (TRANS_A) {
-                const lds_ptr p = base + am_frag[i] + kk * 16 * RB_M;
-                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)p);
-                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * RB_M));
-                u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
-                u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
-                af[i] = u32x4{lo2.x, lo2.y, hi2.x, hi2.y};
-            } else {
-                af[i] = *(const lds_u32x4 *)(base + a_frag + i * 32 * ROW_B + kx[kk]);
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-            if (TRANS_B) {
-                bf[j] = *(const lds_u32x4 *)(base + bt_frag + j * 32 * ROW_B + kx[kk]);
-            } else {
-                const lds_ptr p = base + bn_frag[j] + kk * 16 * RB_N;
-                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)p);
-                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * RB_N));
-                u32x2 lo2 = __builtin_bit_cast(u32x2, lo);
-                u32x2 hi2 = __builtin_bit_cast(u32x2, hi);
-                bf[j] = u32x4{lo2.x, lo2.y, hi2.x, hi2.y};
-            }
+        if constexpr (TRANS_A) {
+            const lds_ptr p = base + am_frag[i] + ks * 32 * RB_M;
+            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)p);
+            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * RB_M));
+            u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+            return u32x4{lo2.x, lo2.y, hi2.x, hi2.y};
+        } else {
+            return *(const lds_u32x4 *)(base + a_frag + i * 16 * ROW_B + kx[ks]);
         }
     };
+    auto read_b = [&](int stage, int ks, int j) -> u32x4 {
+        const lds_ptr base = lds + stage * L::STAGE_BYTES;
+        if constexpr (TRANS_B) {
+            return *(const lds_u32x4 *)(base + bt_frag + j * 16 * ROW_B + kx[ks]);
+        } else {
+            const lds_ptr p = base + bn_frag[j] + ks * 32 * RB_N;
+            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)p);
+            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p + 4 * RB_N));
+            u32x2 lo2 = __builtin_bit_cast(u32x2, lo), hi2 = __builtin_bit_cast(u32x2, hi);
+            return u32x4{lo2.x, lo2.y, hi2.x, hi2.y};
+        }
+    };
+
+    // ---- main loop -----------------------------------------------------------------
+    // At the top of tile kt one barrier establishes two facts: tile kt+1 has landed for every
+    // wave (each waited for its own loads first), and every wave is done reading tile kt-1,
+    // whose stage is refilled right away.  Because tile kt+1 is already complete, the fragments
+    // of its first k-step are read during the last k-step of tile kt: the MFMA queue stays fed
+    // across the barrier.  Tiles kt+2 .. kt+S-1 are in flight meanwhile.  A tile index past the
+    // last one is clamped: the extra loads land in a stage nobody reads again and keep the
+    // number of outstanding loads the same in every iteration, so one constant vmcnt bound
+    // serves the whole loop.
+    //
+    // Inside a k-step the MFMAs run row tile by row tile of A.  The A fragment of row tile i is
+    // dead once its NT products are issued, so the next k-step's fragment for the same row tile
+    // is read into the same registers right behind them; the B fragments are needed by every row
+    // tile and are double buffered.  That keeps a 256x256 tile (128 accumulator registers per
+    // lane) with its fragments inside the 256 registers of a two-waves-per-SIMD workgroup.
+    static_assert(S >= 3, "the ring needs the current, the next and one tile in flight");
+    const int KT = k_len / BK;
+    constexpr int LPS = (LOADS + KS - 1) / KS;  // direct loads issued per k-step
+    constexpr int B_DS = TRANS_B ? 1 : 2, A_DS = TRANS_A ? 2 : 1;  // LDS reads per fragment
 
     s.sync();  // the previous task is done with the stage buffers
 #pragma unroll
@@ -319,86 +349,185 @@ __device__ __forceinline__ void gemm_tile(const GemmDesc &d, int task, const Slo
     wait_vmcnt_then_barrier<(S - 2) * LOADS>();  // tile 0 is complete
 
     u32x4 af[2][MT], bf[2][NT];
-    read_frags(0, 0, af[0], bf[0]);
+#pragma unroll
+    for (int i = 0; i < MT; ++i) af[0][i] = read_a(0, 0, i);
+#pragma unroll
+    for (int j = 0; j < NT; ++j) bf[0][j] = read_b(0, 0, j);
+
     int stage = 0, fill = S - 1;  // fill: the free stage (tile kt-1's), refilled at the top of tile kt
-    constexpr int LPK = (LOADS + KK - 1) / KK;  // direct loads issued per k-step
-    for (int kt = 0; kt < KT; ++kt) {
+    int refill = 0, next_stage = 0;
+    auto tile_top = [&](int kt) {
         wait_vmcnt_then_barrier<(S - 3) * LOADS>();
-        const int refill = min(kt + S - 1, KT - 1);
-        const int next_stage = (stage + 1 == S) ? 0 : stage + 1;
-#pragma unroll
-        for (int kk = 0; kk < KK; ++kk) {
-            // the k-step after this one: the next of this tile, or the first of the next tile
-            if (kk + 1 < KK) read_frags(stage, kk + 1, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-            else read_frags(next_stage, 0, af[(kk + 1) & 1], bf[(kk + 1) & 1]);
-            // this k-step's share of the refill of the stage tile kt-1 used
-#pragma unroll
-            for (int l = kk * LPK; l < (kk + 1) * LPK && l < LOADS; ++l) issue_one(refill, fill, l);
-#pragma unroll
-            for (int i = 0; i < MT; ++i)
-#pragma unroll
-                for (int j = 0; j < NT; ++j)
-                    acc[i][j] = mfma32<T>(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
-            // Issue order: one LDS read or one direct load behind every MFMA.  All
-            // waves leave the barrier together; if each first issued its loads and
-            // reads back to back, they would queue at the CU's one memory pipeline
-            // while the matrix cores wait.
-            // LDS reads first, two behind each MFMA (the next k-step needs all of
-            // them), then the direct loads.
-            constexpr int DS_READS = (TRANS_A ? 2 * MT : MT) + (TRANS_B ? NT : 2 * NT);
-            constexpr int DS_PER = (2 * MT * NT >= DS_READS + 2) ? 2 : (DS_READS + MT * NT - 1) / (MT * NT);
-            constexpr int DS_GROUPS = (DS_READS + DS_PER - 1) / DS_PER;
-            constexpr int VM_GROUPS = (MT * NT > DS_GROUPS) ? MT * NT - DS_GROUPS : 1;
-            constexpr int VM_PER = (LPK + VM_GROUPS - 1) / VM_GROUPS;
-#pragma unroll
-            for (int n = 0; n < MT * NT; ++n) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-                if (n < DS_GROUPS) __builtin_amdgcn_sched_group_barrier(0x100, DS_PER, 0);  // LDS reads
-                if (n >= MT * NT - VM_GROUPS)
-                    __builtin_amdgcn_sched_group_barrier(0x020, VM_PER, 0);  // direct loads
-            }
-        }
+        refill = min(kt + S - 1, KT - 1);
+        next_stage = (stage + 1 == S) ? 0 : stage + 1;
+    };
+    auto tile_end = [&]() {
         stage = next_stage;
         fill = (fill + 1 == S) ? 0 : fill + 1;
+    };
+    // One k-step multiplies fragment set CUR and reads set CUR^1 for the k-step after it.  The
+    // MFMAs run row tile by row tile of A; the reads of the next set are dealt to the first row
+    // tiles (the next step's first operands first) and the last two row tiles read nothing, so
+    // that every read has returned when the step ends at the barrier.  Row tile I's part
+    // (compile-time I: the scheduling hints take constants only):
+    constexpr int NREADS = MT + NT;              // fragments per k-step
+    constexpr int NRT = MT > 2 ? MT - 2 : 1;     // row tiles that issue reads
+    auto read_one = [&](auto cur_c, auto r_c, int nstage, int nks) {
+        constexpr int CUR = decltype(cur_c)::value, R = decltype(r_c)::value;
+        // read order: a0, b0 .. b(NT-1), a1 .. a(MT-1)
+        if constexpr (R == 0) af[CUR ^ 1][0] = read_a(nstage, nks, 0);
+        else if constexpr (R <= NT) bf[CUR ^ 1][R - 1] = read_b(nstage, nks, R - 1);
+        else af[CUR ^ 1][R - NT] = read_a(nstage, nks, R - NT);
+    };
+    auto row_tile = [&](auto cur_c, auto ks_c, auto i_c, int nstage, int nks) {
+        constexpr int CUR = decltype(cur_c)::value, KS_I = decltype(ks_c)::value, I = decltype(i_c)::value;
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[I][j] = mfma16x32<T>(bf[CUR][j], af[CUR][I], acc[I][j]);
+        constexpr int R0 = I < NRT ? (I * NREADS) / NRT : NREADS, R1 = I < NRT ? ((I + 1) * NREADS) / NRT : NREADS;
+        static_for<R1 - R0>([&](auto r_c) {
+            read_one(cur_c, std::integral_constant<int, R0 + decltype(r_c)::value>{}, nstage, nks);
+        });
+        // LDS instructions of those reads: fragment r is b(r-1) for 1 <= r <= NT, else an A fragment
+        constexpr int NB = (R1 < NT + 1 ? R1 : NT + 1) - (R0 > 1 ? (R0 < NT + 1 ? R0 : NT + 1) : (R1 >= 1 ? 1 : R1));
+        constexpr int NB_ = NB > 0 ? NB : 0;
+        constexpr int DS = NB_ * B_DS + (R1 - R0 - NB_) * A_DS;
+        // this row tile's share of the refill of the stage tile kt-1 used
+        constexpr int L0 = KS_I * LPS + (I * LPS) / MT, L1 = KS_I * LPS + ((I + 1) * LPS) / MT;
+        constexpr int LB = L0 < LOADS ? L0 : LOADS, LE = L1 < LOADS ? L1 : LOADS;
+#pragma unroll
+        for (int l = LB; l < LE; ++l) issue_one(refill, fill, l);
+        // Issue order: the LDS reads and direct loads of a row tile sit between its MFMAs.  All
+        // waves leave the barrier together; if each first issued its loads and reads back to
+        // back, they would queue at the CU's one memory pipeline while the matrix cores wait.
+        constexpr int HEAD = NT >= 2 ? NT / 2 : NT;
+        __builtin_amdgcn_sched_group_barrier(0x008, HEAD, 0);  // MFMA
+        if constexpr (DS > 0) __builtin_amdgcn_sched_group_barrier(0x100, DS, 0);  // LDS reads
+        if constexpr (NT - HEAD > 0) __builtin_amdgcn_sched_group_barrier(0x008, NT - HEAD, 0);
+        if constexpr (LE - LB > 0) __builtin_amdgcn_sched_group_barrier(0x020, LE - LB, 0);  // direct loads
+    };
+    auto kstep = [&](auto cur_c, auto ks_c) {
+        constexpr int KS_I = decltype(ks_c)::value;
+        constexpr bool last = (KS_I + 1 == KS);
+        const int nstage = last ? next_stage : stage;
+        constexpr int nks = last ? 0 : KS_I + 1;
+        static_for<MT>([&](auto i_c) { row_tile(cur_c, ks_c, i_c, nstage, nks); });
+    };
+    using std::integral_constant;
+    if constexpr (KS == 1) {
+        // the B buffers alternate from tile to tile: two tiles per trip (K is a multiple of 64)
+        for (int kt = 0; kt < KT; kt += 2) {
+            tile_top(kt);
+            kstep(integral_constant<int, 0>{}, integral_constant<int, 0>{});
+            tile_end();
+            tile_top(kt + 1);
+            kstep(integral_constant<int, 1>{}, integral_constant<int, 0>{});
+            tile_end();
+        }
+    } else {
+        static_assert(KS == 2, "K tiles are 32 or 64 deep");
+        for (int kt = 0; kt < KT; ++kt) {
+            tile_top(kt);
+            kstep(integral_constant<int, 0>{}, integral_constant<int, 0>{});
+            kstep(integral_constant<int, 1>{}, integral_constant<int, 1>{});
+            tile_end();
+        }
     }
     // the clamped loads still in flight target LDS: they must land before the
     // buffers are used again (by the next task or another op body)
     wait_vmcnt_then_barrier<0>();
 
-    // ---- epilogue: C fragment row = 8*(r/4) + 4*(lane/32) + r%4, col = lane%32 --
+    if constexpr (SPLIT) {
+        // Partials travel as agent-scope relaxed atomics (write-through stores, L2-bypassing
+        // loads): the two halves run on different XCDs, whose L2s do not see each other.
+        // Ordering: every wave waits for its stores to be acknowledged before the workgroup
+        // barrier, the arrival is counted after it, and the other half's partials are read only
+        // by the workgroup that saw the count at one.
+        constexpr int PER_THREAD = MT * NT;  // f32x4 values
+        const int64_t tile_words = (int64_t)2 * kGemmThreads * PER_THREAD * 4;
+        float *mine = d.partial + (int64_t)task * tile_words + ((int64_t)half * kGemmThreads + tid) * PER_THREAD * 4;
+        float *theirs = d.partial + (int64_t)task * tile_words + ((int64_t)(half ^ 1) * kGemmThreads + tid) * PER_THREAD * 4;
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                uint64_t w[2];
+                __builtin_memcpy(w, &acc[i][j], 16);
+                uint64_t *p = reinterpret_cast<uint64_t *>(mine + (i * NT + j) * 4);
+                __hip_atomic_store(p, w[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(p + 1, w[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        drain_stores_then_barrier();
+        lds_i32x *flag = (lds_i32x *)lds;
+        if (tid == 0)
+            *flag = (int)__hip_atomic_fetch_add(d.arrivals + task, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s.sync();
+        const int arrived_before = *flag;
+        s.sync();  // the flag word is part of the stage buffers the next task refills
+        if (arrived_before == 0) return -1;
+        if (tid == 0) __hip_atomic_store(d.arrivals + task, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+        for (int i = 0; i < MT; ++i)
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                const uint64_t *p = reinterpret_cast<const uint64_t *>(theirs + (i * NT + j) * 4);
+                uint64_t w[2] = {__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
+                                 __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)};
+                f32x4 o;
+                __builtin_memcpy(&o, w, 16);
+                acc[i][j] += o;
+            }
+    }
+
+    // ---- epilogue: lane (m = lane%16, g = lane/16) holds C[m][4g .. 4g+3] of each 16x16 tile ----
+    const bool vec_ok = ((d.ldc & 3) == 0) && (((uintptr_t)d.c & 7) == 0) && ((d.c_bs[0] & 3) == 0) &&
+                        ((d.c_bs[1] & 3) == 0);
+    auto store4 = [&](int row, int col, float v0, float v1, float v2, float v3) {
+        if (row >= d.store_m) return;
+        gptr<T> p = C + (int64_t)row * d.ldc + col;
+        if (vec_ok && col + 4 <= d.store_n) {
+            T o[4] = {from_f32<T>(epi(v0, row, col)), from_f32<T>(epi(v1, row, col + 1)),
+                      from_f32<T>(epi(v2, row, col + 2)), from_f32<T>(epi(v3, row, col + 3))};
+            u32x2 w;
+            __builtin_memcpy(&w, o, 8);
+            *(ARKMI_GLOBAL u32x2 *)p = w;
+        } else {
+            const float v[4] = {v0, v1, v2, v3};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col + e < d.store_n) p[e] = from_f32<T>(epi(v[e], row, col + e));
+        }
+    };
     if constexpr (DUAL_B) {
-        // accumulator tiles 2p and 2p+1 of a wave hold the gate and the up product of the
-        // same 32 output columns
+        // accumulator tiles j and j + NT/2 of a wave hold the gate and the up product of the
+        // same 16 output columns
         static_assert(NT % 2 == 0, "the gate/up pair needs an even number of column tiles per wave");
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
+            const int row = m0 + wm * WTM + i * 16 + l16;
 #pragma unroll
-            for (int p = 0; p < NT / 2; ++p) {
-                const int col = tn * (BN / 2) + wn * (WTN / 2) + p * 32 + (lane & 31);
+            for (int j = 0; j < NT / 2; ++j) {
+                const int col = tn * (BN / 2) + wn * (WTN / 2) + j * 16 + 4 * g4;
+                float o[4];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                    const float g = acc[i][2 * p][r], u = acc[i][2 * p + 1][r];
-                    if (row < d.store_m && col < d.store_n)
-                        C[(int64_t)row * d.ldc + col] = from_f32<T>(epi(g / (1.f + __expf(-g)) * u, row, col));
+                for (int e = 0; e < 4; ++e) {
+                    const float g = acc[i][j][e], u = acc[i][j + NT / 2][e];
+                    o[e] = g / (1.f + __expf(-g)) * u;
                 }
+                store4(row, col, o[0], o[1], o[2], o[3]);
             }
         }
-        return;
+        return task;
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
+        const int row = m0 + wm * WTM + i * 16 + l16;
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
-            const int col = n0 + wn * WTN + j * 32 + (lane & 31);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int row = m0 + wm * WTM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-                if (row < d.store_m && col < d.store_n)
-                    C[(int64_t)row * d.ldc + col] = from_f32<T>(epi(acc[i][j][r], row, col));
-            }
+            const int col = n0 + wn * WTN + j * 16 + 4 * g4;
+            store4(row, col, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
         }
     }
+    return task;
 }
 
 }  // namespace arkmi

@@ -28,8 +28,10 @@ enum DevOpKind : int32_t { DEV_NOOP = 0, DEV_ROW = 1, DEV_GEMM = 2, DEV_EWISE = 
 // FAM_EXT holds the bodies few plans use (fp32 and transposed-first-operand matmuls,
 // reductions over an axis other than the last, the embedding gather): kept out of the common variants, whose
 // register allocation and code size every other body shares.
+// FAM_SPLITK adds the matmul body that splits K in two (256x256 tiles only) to a variant
+// that carries FAM_GEMM.
 enum OpFamily : int32_t { FAM_ROW = 1, FAM_EWISE = 2, FAM_GEMM = 4, FAM_GEMV = 8, FAM_ATTN = 16, FAM_EXT = 32,
-                          FAM_ALL = 63 };
+                          FAM_SPLITK = 64, FAM_ALL = 127 };
 
 struct DevOp {
     int32_t kind;

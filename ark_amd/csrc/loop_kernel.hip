@@ -19,7 +19,11 @@ const void *loop_kernel_variant_16();  // attention
 const void *loop_kernel_variant_23();  // rows + elementwise + GEMM + attention
 const void *loop_kernel_variant_31();  // every common family
 const void *loop_kernel_variant_32();  // the rarely used bodies alone
-const void *loop_kernel_variant_63();  // everything
+const void *loop_kernel_variant_63();  // everything but the split of K
+const void *loop_kernel_variant_68();  // GEMM incl. the split of K
+const void *loop_kernel_variant_70();  // elementwise + GEMM incl. the split of K
+const void *loop_kernel_variant_87();  // rows + elementwise + GEMM incl. the split of K + attention
+const void *loop_kernel_variant_127(); // everything
 
 const void *step_kernel_variant_1();
 const void *step_kernel_variant_2();
@@ -29,6 +33,7 @@ const void *step_kernel_variant_6();
 const void *step_kernel_variant_8();
 const void *step_kernel_variant_16();
 const void *step_kernel_variant_32();
+const void *step_kernel_variant_70();
 
 const void *step_kernel_select(int families) {
     struct Variant { int fam; const void *(*get)(); };
@@ -36,6 +41,7 @@ const void *step_kernel_select(int families) {
         {1, step_kernel_variant_1}, {2, step_kernel_variant_2}, {8, step_kernel_variant_8}, {16, step_kernel_variant_16},
         {32, step_kernel_variant_32},
         {3, step_kernel_variant_3}, {4, step_kernel_variant_4}, {6, step_kernel_variant_6},
+        {70, step_kernel_variant_70},
     };
     for (const Variant &v : table)
         if ((families & ~v.fam) == 0) return v.get();
@@ -58,6 +64,8 @@ const void *loop_kernel_select(int families, int *chosen) {
         {3, loop_kernel_variant_3},   {11, loop_kernel_variant_11}, {4, loop_kernel_variant_4},
         {6, loop_kernel_variant_6},   {7, loop_kernel_variant_7},   {23, loop_kernel_variant_23},
         {31, loop_kernel_variant_31}, {63, loop_kernel_variant_63},
+        {68, loop_kernel_variant_68}, {70, loop_kernel_variant_70}, {87, loop_kernel_variant_87},
+        {127, loop_kernel_variant_127},
     };
     for (const Variant &v : table) {
         if ((families & ~v.fam) == 0) {
@@ -66,7 +74,7 @@ const void *loop_kernel_select(int families, int *chosen) {
         }
     }
     if (chosen) *chosen = FAM_ALL;
-    return loop_kernel_variant_63();
+    return loop_kernel_variant_127();
 }
 
 void loop_kernel_prepare(const void *kernel, int lds_bytes) {

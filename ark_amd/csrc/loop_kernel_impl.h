@@ -164,21 +164,28 @@ __device__ __forceinline__ D load_const(const D *p) {
     return d;
 }
 
-template <typename T, bool TRANS_B>
-__device__ __forceinline__ void gemm_by_tile(const DevOp *op, int task, const Slot &s) {
+// Returns the task index the ops fused behind the matmul run for (the tile this workgroup
+// finished), -1 when another workgroup finishes the tile (a split of K).
+template <int FAM, typename T, bool TRANS_B>
+__device__ __forceinline__ int gemm_by_tile(const DevOp *op, int task, const Slot &s) {
     const GemmDesc g = load_const(&op->gemm);
     const int tm = load_const(&op->gemm_tile_m), tn = load_const(&op->gemm_tile_n);
+    if (g.split_k == 2) {  // 256x256 tiles only (checked on the host)
+        if constexpr ((FAM & FAM_SPLITK) != 0)
+            return gemm_tile<T, 256, 256, TRANS_B, EpilogueStore, false, false, true>(g, task, s, EpilogueStore());
+        else
+            return -1;
+    }
     if constexpr (TRANS_B) {
         if (g.b2) {  // gate/up pair: 256-wide tiles only (checked on the host)
-            if (tm == 256) gemm_tile<T, 256, 256, true, EpilogueStore, false, true>(g, task, s, EpilogueStore());
-            else gemm_tile<T, 128, 256, true, EpilogueStore, false, true>(g, task, s, EpilogueStore());
-            return;
+            if (tm == 256) return gemm_tile<T, 256, 256, true, EpilogueStore, false, true>(g, task, s, EpilogueStore());
+            return gemm_tile<T, 128, 256, true, EpilogueStore, false, true>(g, task, s, EpilogueStore());
         }
     }
-    if (tm == 256 && tn == 256) gemm_tile<T, 256, 256, TRANS_B>(g, task, s, EpilogueStore());
-    else if (tm == 128 && tn == 256) gemm_tile<T, 128, 256, TRANS_B>(g, task, s, EpilogueStore());
-    else if (tm == 256 && tn == 128) gemm_tile<T, 256, 128, TRANS_B>(g, task, s, EpilogueStore());
-    else gemm_tile<T, 128, 128, TRANS_B>(g, task, s, EpilogueStore());
+    if (tm == 256 && tn == 256) return gemm_tile<T, 256, 256, TRANS_B>(g, task, s, EpilogueStore());
+    if (tm == 128 && tn == 256) return gemm_tile<T, 128, 256, TRANS_B>(g, task, s, EpilogueStore());
+    if (tm == 256 && tn == 128) return gemm_tile<T, 256, 128, TRANS_B>(g, task, s, EpilogueStore());
+    return gemm_tile<T, 128, 128, TRANS_B>(g, task, s, EpilogueStore());
 }
 
 // FAM is the set of op families compiled into this kernel variant.  The families
@@ -187,8 +194,10 @@ __device__ __forceinline__ void gemm_by_tile(const DevOp *op, int task, const Sl
 // register allocation, and the row and elementwise bodies then spill values
 // that live across the task loop and reload them in their inner loops.  A
 // plan runs on the smallest variant that holds its families.
+// Returns the task index for the ops that follow in the same fused task: `task` itself, except
+// behind a matmul that splits K, where it is the tile this workgroup finished or -1 (none).
 template <int FAM>
-__device__ __forceinline__ void run_op(const DevOp *op, int task, const Slot &s_in) {
+__device__ __forceinline__ int run_op(const DevOp *op, int task, const Slot &s_in) {
     // For the long-running bodies the thread index is made opaque per task: the per-lane
     // addresses they derive from it would otherwise be hoisted out of the task and step
     // loops as invariants and stay in registers across every other body.  The short
@@ -230,11 +239,11 @@ __device__ __forceinline__ void run_op(const DevOp *op, int task, const Slot &s_
             } else if constexpr ((FAM & FAM_GEMM) != 0) {
                 const bool trans_b = load_const(&op->gemm.trans_b) != 0;
                 if (load_const(&op->gemm.dtype) == 1) {
-                    if (trans_b) gemm_by_tile<f16, true>(op, task, s);
-                    else gemm_by_tile<f16, false>(op, task, s);
+                    if (trans_b) return gemm_by_tile<FAM, f16, true>(op, task, s);
+                    return gemm_by_tile<FAM, f16, false>(op, task, s);
                 } else {
-                    if (trans_b) gemm_by_tile<bf16, true>(op, task, s);
-                    else gemm_by_tile<bf16, false>(op, task, s);
+                    if (trans_b) return gemm_by_tile<FAM, bf16, true>(op, task, s);
+                    return gemm_by_tile<FAM, bf16, false>(op, task, s);
                 }
             }
             break;
@@ -258,6 +267,7 @@ __device__ __forceinline__ void run_op(const DevOp *op, int task, const Slot &s_
             break;
         default: break;
     }
+    return task;
 }
 
 // task_seq<> of the reference, parameters read from the table
@@ -300,7 +310,8 @@ __device__ __forceinline__ void run_group(const LoopProgram &prog, const DevTask
             prog.trace[g.trace_offset + (int)((id - g.task_b) / g.task_s)] = rec;
         }
 #endif
-        for (int o = 0; o < g.op_count; ++o) {
+        int follow = (int)id;  // uniform across the workgroup
+        for (int o = 0; o < g.op_count && follow >= 0; ++o) {
             if (o > 0) {
                 // later ops of a fused task read what earlier ones wrote: the stores
                 // have reached the L2, and the L1 must not serve older copies
@@ -308,7 +319,7 @@ __device__ __forceinline__ void run_group(const LoopProgram &prog, const DevTask
                 if (s.tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
                 s.sync();
             }
-            run_op<FAM>(ops + o, (int)id, s);
+            follow = run_op<FAM>(ops + o, follow, s);
         }
     }
 }

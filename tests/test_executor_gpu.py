@@ -852,3 +852,64 @@ def test_cast_through_bytes(oracle, dtype):
     assert np.array_equal(g_t.view(np.uint8), raw) and g_t.shape == want.shape
     assert np.array_equal(g_back, raw)
     assert np.array_equal(g_copy.view(np.uint8).reshape(raw.shape), raw)
+
+
+# ---------------------------------------------------------------- matmul with K split in two
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("trans_other", [False, True])
+def test_matmul_split_k(oracle, dtype, trans_other):
+    """An output that gives 256x256 tiles to half of the CUs only (2048 x 4096, the decoder layer's
+    projections) is planned with SplitK 2: two tasks per tile, each multiplying half of K; the half
+    that finishes second adds the two.  Several iterations reuse the arrival counters; checked on
+    sampled rows against the oracle, and bit for bit against the same plan run one kernel per op."""
+    import torch
+    from ark_amd import Model, Executor
+    M, N, K = 2048, 4096, 2048
+    a = make(oracle, (M, K), dtype, 111, "uniform")
+    b = make(oracle, (N, K) if trans_other else (K, N), dtype, 112, "normal", scale=0.05)
+    m = Model()
+    ta, tb = m.tensor(a.shape, dtype), m.tensor(b.shape, dtype)
+    c = m.matmul(ta, tb, trans_other=trans_other)
+    plan = m.plan(device_id=0)
+    cfg = json.loads(plan)["TaskInfos"][0]["Ops"][0]["Config"]
+    assert cfg["SplitK"] == 2 and cfg["TileShapeMNK"][:2] == [256, 256] and cfg["NumTasks"] == 2 * 8 * 16, cfg
+    (got,), ex, _ = run_model(m, {ta: a, tb: b}, [c], iters=3, plan=plan)
+    assert ex.info()["iteration_sync"] == 2 and (ex.info()["kernel_families"] & 64), ex.info()
+    pick = np.sort(np.random.default_rng(5).choice(M, 32, replace=False))
+    pick[0], pick[-1] = 0, M - 1
+    close(oracle, oracle.matmul(np.ascontiguousarray(a[pick]), b, dtype, trans_b=trans_other), got[pick], dtype, 1e-2)
+    ex2 = Executor(plan, device_id=0, loop_mode=False).compile()
+    ex2.tensor_write(ta, a)
+    ex2.tensor_write(tb, b)
+    ex2.run_separate(2)
+    torch.cuda.synchronize()
+    assert np.array_equal(ex2.tensor_read(c), got)
+
+
+def test_matmul_split_k_with_follower_and_neighbours(oracle):
+    """The residual add fused behind a split matmul runs on the workgroup that finishes the tile; the
+    ops before and after it keep their grid barriers (a split tile has no fixed workgroup)."""
+    from ark_amd import Model
+    dtype = "bf16"
+    M, N, K = 2048, 4096, 2048
+    x = make(oracle, (M, K), dtype, 113, "normal")
+    w = make(oracle, (N, K), dtype, 114, "normal", scale=0.02)
+    r = make(oracle, (M, N), dtype, 115, "normal")
+    m = Model()
+    tx, tw, tr = m.tensor(x.shape, dtype), m.tensor(w.shape, dtype), m.tensor(r.shape, dtype)
+    xs = m.mul(tx, 0.5)
+    with m.planner_context(sync=False):
+        h = m.add(tr, m.matmul(xs, tw, trans_other=True))
+    out = m.relu(h)
+    plan = m.plan(device_id=0)
+    tasks = json.loads(plan)["TaskInfos"]
+    assert len(tasks) == 3 and len(tasks[1]["Ops"]) == 2 and tasks[1]["Ops"][0]["Config"].get("SplitK") == 2
+    assert tasks[1]["Ops"][1]["Config"]["NumTasks"] * 2 == tasks[1]["Ops"][0]["Config"]["NumTasks"]
+    (got,), ex, _ = run_model(m, {tx: x, tw: w, tr: r}, [out], iters=2, plan=plan)
+    assert ex.info()["barriers_local"] == 0 and ex.info()["barriers_elided"] == 0, ex.info()
+    pick = np.sort(np.random.default_rng(6).choice(M, 24, replace=False))
+    pick[0], pick[-1] = 0, M - 1
+    xs_ref = oracle.scalar(np.ascontiguousarray(x[pick]), 0.5, "mul", dtype)
+    ref = oracle.unary(oracle.binary(np.ascontiguousarray(r[pick]), oracle.matmul(xs_ref, w, dtype, trans_b=True),
+                                     "add", dtype), "relu", dtype)
+    close(oracle, ref, got[pick], dtype, 1e-2)

@@ -349,7 +349,8 @@ def test_rocm950_matmul_tile_choice():
         c = json.loads(m.plan(arch="ROCM_950", num_processors=256))["TaskInfos"][0]["Ops"][0]["Config"]
         return c["TileShapeMNK"][:2], c["NumTasks"]
     assert tile(8192, 11008, 4096) == ([256, 256], 32 * 43)
-    assert tile(2048, 4096, 4096) == ([128, 256], 16 * 16)        # 256x256 would leave CUs idle
+    assert tile(2048, 4096, 4096) == ([256, 256], 2 * 8 * 16)     # 128 large tiles, K split in two
+    assert tile(2048, 4096, 1024) == ([128, 256], 16 * 16)        # short K: smaller tiles instead
     assert tile(2048, 2048, 128, batch=(1, 32)) == ([256, 256], 32 * 64)
     assert tile(512, 512, 64) == ([128, 128], 16)
     with pytest.raises(ArkmiError) as e:
@@ -382,3 +383,25 @@ def test_follower_takes_producer_tiles_through_a_reshape():
         m.mul(y, g)
     plan = json.loads(m.plan(arch="ROCM_950", num_processors=256))
     assert "ViewAs" not in plan["TaskInfos"][0]["Ops"][1]["Config"]
+
+
+def test_rocm950_matmul_tiles_and_split_k():
+    """The gfx950 default rule: the largest tile that still gives every CU a task; an output that
+    gives 256x256 tiles to between half and all of the CUs keeps them and splits K in two."""
+    def cfg(M, N, K, ncu=256, trans_other=False):
+        m = Model()
+        a, b = m.tensor([M, K], "bf16"), m.tensor([N, K] if trans_other else [K, N], "bf16")
+        m.matmul(a, b, trans_other=trans_other)
+        return json.loads(m.plan(arch="ROCM_950", num_processors=ncu))["TaskInfos"][0]["Ops"][0]["Config"]
+    c = cfg(4096, 4096, 4096)
+    assert c["TileShapeMNK"][:2] == [256, 256] and c["NumTasks"] == 256 and "SplitK" not in c
+    c = cfg(2048, 4096, 4096, trans_other=True)
+    assert c["TileShapeMNK"][:2] == [256, 256] and c["SplitK"] == 2 and c["NumTasks"] == 256
+    c = cfg(2048, 4096, 11008, trans_other=True)
+    assert c["SplitK"] == 2 and c["NumTasks"] == 256
+    c = cfg(2048, 4096, 1024)                       # short K: not worth splitting
+    assert "SplitK" not in c and c["NumTasks"] >= 256
+    c = cfg(2048, 2048, 4096)                       # 64 large tiles: smaller tiles fill the chip instead
+    assert "SplitK" not in c and c["TileShapeMNK"][:2] == [128, 128]
+    c = cfg(2048, 4096, 4096, ncu=128)              # a plan for 128 processors has a tile for each already
+    assert "SplitK" not in c and c["TileShapeMNK"][:2] == [256, 256] and c["NumTasks"] == 128
