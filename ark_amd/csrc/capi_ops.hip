@@ -331,3 +331,76 @@ extern "C" int arkmi_gemv_static(int dtype, const void *x, const void *w, void *
         launch_gemv(dtype, x, w, y, m, n, k, ldx, ldw, ldy, num_tasks, ws, st);
     });
 }
+
+// ---- measurement probes: what the machine sustains, beside the datasheet peaks ------
+namespace arkmi {
+
+// Every wave runs `iters` rounds of 16 independent v_mfma_f32_16x16x32_f16 on operand registers
+// loaded from `operands` (random data draws more power than zeros, and the chip clocks down).
+__global__ __launch_bounds__(kBlock) void probe_mfma_kernel(const u32x4 *operands, int iters, float *sink) {
+    u32x4 a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a[i] = operands[(threadIdx.x + i * kBlock) & 65535];
+        b[i] = operands[(threadIdx.x + i * kBlock + 7777) & 65535];
+    }
+    f32x4 acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = mfma16x32<f16>(a[i & 3], b[i >> 2], acc[i]);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s += acc[i][0] + acc[i][1] + acc[i][2] + acc[i][3];
+    if (s == 1234567.f) sink[0] = s;  // keeps the loop alive
+}
+
+// Streams `bytes` from src as 16-byte vectors, 4 in flight per thread; writes them to dst when
+// given (a copy), else folds them into a value that is (practically never) stored.
+__global__ __launch_bounds__(256) void probe_stream_kernel(const u32x4 *src, u32x4 *dst, size_t n_vec, uint32_t *sink) {
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    u32x4 acc = {0, 0, 0, 0};
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += 4 * stride) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (i + u * stride < n_vec) v[u] = __builtin_nontemporal_load(src + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (i + u * stride < n_vec) {
+                if (dst) __builtin_nontemporal_store(v[u], dst + i + u * stride);
+                else acc ^= v[u];
+            }
+    }
+    if (!dst && (acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = acc.x;
+}
+
+}  // namespace arkmi
+
+extern "C" int arkmi_probe_mfma(const void *operands, size_t operand_bytes, int iters, void *sink, double *flops,
+                                void *stream) {
+    return guard([&] {
+        if (!operands || !sink || operand_bytes < (size_t)65536 * 16)
+            ARKMI_FAIL(ARKMI_INVALID_USAGE, "the MFMA probe reads 1 MiB of operand data and needs a 4-byte sink");
+        if (iters < 1) ARKMI_FAIL(ARKMI_INVALID_USAGE, "iters must be positive");
+        const int grid = device_facts(current_device()).num_cu;
+        hipLaunchKernelGGL(probe_mfma_kernel, dim3(grid), dim3(kBlock), 0, (hipStream_t)stream,
+                           static_cast<const u32x4 *>(operands), iters, static_cast<float *>(sink));
+        ARKMI_HIP(hipGetLastError());
+        if (flops) *flops = (double)grid * (kBlock / 64) * (double)iters * 16.0 * (2.0 * 16 * 16 * 32);
+    });
+}
+
+extern "C" int arkmi_probe_stream(const void *src, void *dst, size_t bytes, void *sink, void *stream) {
+    return guard([&] {
+        if (!src || !sink || (bytes % 16) || ((uintptr_t)src & 15) || ((uintptr_t)dst & 15))
+            ARKMI_FAIL(ARKMI_INVALID_USAGE, "the stream probe takes 16-byte aligned buffers of whole 16-byte vectors");
+        const int grid = device_facts(current_device()).num_cu * 8;
+        hipLaunchKernelGGL(probe_stream_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream,
+                           static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), bytes / 16,
+                           static_cast<uint32_t *>(sink));
+        ARKMI_HIP(hipGetLastError());
+    });
+}

@@ -56,7 +56,7 @@ struct GemmDesc {
     // that arrives second adds the other's and finishes the tile.  Nobody waits.
     int32_t split_k;           // 1 or 2
     int32_t pad_;
-    float *partial;            // [tiles][2][512 threads][MT * NT] x 4 floats
+    float *partial;            // [tiles][2 halves][MT * NT][512 threads] x 4 floats
     unsigned int *arrivals;    // [tiles], zero between uses
 };
 
@@ -333,11 +333,6 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     // number of outstanding loads the same in every iteration, so one constant vmcnt bound
     // serves the whole loop.
     //
-    // Inside a k-step the MFMAs run row tile by row tile of A.  The A fragment of row tile i is
-    // dead once its NT products are issued, so the next k-step's fragment for the same row tile
-    // is read into the same registers right behind them; the B fragments are needed by every row
-    // tile and are double buffered.  That keeps a 256x256 tile (128 accumulator registers per
-    // lane) with its fragments inside the 256 registers of a two-waves-per-SIMD workgroup.
     static_assert(S >= 3, "the ring needs the current, the next and one tile in flight");
     const int KT = k_len / BK;
     constexpr int LPS = (LOADS + KS - 1) / KS;  // direct loads issued per k-step
@@ -348,9 +343,10 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     for (int p = 0; p < S - 1; ++p) issue(min(p, KT - 1), p);
     wait_vmcnt_then_barrier<(S - 2) * LOADS>();  // tile 0 is complete
 
-    u32x4 af[2][MT], bf[2][NT];
+    constexpr int A_SET = (MT >= 8 && NT >= 4) ? MT / 2 : MT;  // A fragments per register set (see below)
+    u32x4 af[2][A_SET], bf[2][NT];
 #pragma unroll
-    for (int i = 0; i < MT; ++i) af[0][i] = read_a(0, 0, i);
+    for (int i = 0; i < A_SET; ++i) af[0][i] = read_a(0, 0, i);
 #pragma unroll
     for (int j = 0; j < NT; ++j) bf[0][j] = read_b(0, 0, j);
 
@@ -365,37 +361,58 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
         stage = next_stage;
         fill = (fill + 1 == S) ? 0 : fill + 1;
     };
-    // One k-step multiplies fragment set CUR and reads set CUR^1 for the k-step after it.  The
-    // MFMAs run row tile by row tile of A; the reads of the next set are dealt to the first row
-    // tiles (the next step's first operands first) and the last two row tiles read nothing, so
-    // that every read has returned when the step ends at the barrier.  Row tile I's part
-    // (compile-time I: the scheduling hints take constants only):
-    constexpr int NREADS = MT + NT;              // fragments per k-step
-    constexpr int NRT = MT > 2 ? MT - 2 : 1;     // row tiles that issue reads
-    auto read_one = [&](auto cur_c, auto r_c, int nstage, int nks) {
-        constexpr int CUR = decltype(cur_c)::value, R = decltype(r_c)::value;
-        // read order: a0, b0 .. b(NT-1), a1 .. a(MT-1)
-        if constexpr (R == 0) af[CUR ^ 1][0] = read_a(nstage, nks, 0);
-        else if constexpr (R <= NT) bf[CUR ^ 1][R - 1] = read_b(nstage, nks, R - 1);
-        else af[CUR ^ 1][R - NT] = read_a(nstage, nks, R - NT);
+    // A k-step of a 256x256 tile runs in two phases, the upper and the lower half of the wave's
+    // row tiles (PH = 2).  Phase H multiplies A fragment set H by the k-step's B fragments (set
+    // CUR) and meanwhile reads A set H^1 for the phase after it plus half of the next k-step's B
+    // fragments (set CUR^1): 16 fragments in registers instead of 24, which is what lets the body
+    // share a kernel with others without spilling.  Smaller tiles run a k-step as one phase
+    // (PH = 1) that reads the whole next k-step (their phases would be too short to cover the
+    // LDS latency).  The reads are issued in the phase's first row tiles, the next phase's first
+    // operands first, and its last row tile reads nothing, so every read has returned when the
+    // phase ends (also at the barrier on top of a K tile).
+    constexpr int PH = (MT >= 8 && NT >= 4) ? 2 : 1;
+    constexpr int MH = MT / PH;              // row tiles per phase
+    constexpr int NBH = (NT + PH - 1) / PH;  // B fragments read per phase
+    constexpr int NREADS = MH + NBH;         // fragments read per phase
+    constexpr int NRT = MH > 2 ? MH - (PH == 2 ? 1 : 2) : 1;  // row tiles of a phase that issue reads
+    static_assert(MT % PH == 0, "the wave's row tiles split evenly over the phases");
+    // fragment read R of phase H: a0 first, then the phase's B fragments, then the other A fragments
+    auto read_one = [&](auto cur_c, auto h_c, auto r_c, int astage, int aks, int bstage, int bks) {
+        constexpr int CUR = decltype(cur_c)::value, H = decltype(h_c)::value, R = decltype(r_c)::value;
+        constexpr int ASET = PH == 2 ? (H ^ 1) : (CUR ^ 1);      // the A set being filled
+        constexpr int AROW = PH == 2 ? (H ^ 1) * MH : 0;          // its first row tile
+        constexpr int BJ0 = H * NBH;                              // first B fragment this phase reads
+        if constexpr (R == 0) {
+            af[ASET][0] = read_a(astage, aks, AROW);
+        } else if constexpr (R <= NBH) {
+            if constexpr (BJ0 + R - 1 < NT) bf[CUR ^ 1][BJ0 + R - 1] = read_b(bstage, bks, BJ0 + R - 1);
+        } else {
+            af[ASET][R - NBH] = read_a(astage, aks, AROW + R - NBH);
+        }
     };
-    auto row_tile = [&](auto cur_c, auto ks_c, auto i_c, int nstage, int nks) {
-        constexpr int CUR = decltype(cur_c)::value, KS_I = decltype(ks_c)::value, I = decltype(i_c)::value;
+    auto row_tile = [&](auto cur_c, auto ks_c, auto h_c, auto i_c, int astage, int aks, int bstage, int bks) {
+        constexpr int CUR = decltype(cur_c)::value, KS_I = decltype(ks_c)::value, H = decltype(h_c)::value,
+                      I = decltype(i_c)::value;
+        constexpr int ASET = PH == 2 ? H : CUR;
 #pragma unroll
-        for (int j = 0; j < NT; ++j) acc[I][j] = mfma16x32<T>(bf[CUR][j], af[CUR][I], acc[I][j]);
+        for (int j = 0; j < NT; ++j) acc[H * MH + I][j] = mfma16x32<T>(bf[CUR][j], af[ASET][I], acc[H * MH + I][j]);
         constexpr int R0 = I < NRT ? (I * NREADS) / NRT : NREADS, R1 = I < NRT ? ((I + 1) * NREADS) / NRT : NREADS;
         static_for<R1 - R0>([&](auto r_c) {
-            read_one(cur_c, std::integral_constant<int, R0 + decltype(r_c)::value>{}, nstage, nks);
+            read_one(cur_c, h_c, std::integral_constant<int, R0 + decltype(r_c)::value>{}, astage, aks, bstage, bks);
         });
-        // LDS instructions of those reads: fragment r is b(r-1) for 1 <= r <= NT, else an A fragment
-        constexpr int NB = (R1 < NT + 1 ? R1 : NT + 1) - (R0 > 1 ? (R0 < NT + 1 ? R0 : NT + 1) : (R1 >= 1 ? 1 : R1));
-        constexpr int NB_ = NB > 0 ? NB : 0;
-        constexpr int DS = NB_ * B_DS + (R1 - R0 - NB_) * A_DS;
+        // LDS instructions of those reads
+        constexpr int DS = [&]() constexpr {
+            int n = 0;
+            for (int r = R0; r < R1; ++r)
+                n += (r == 0 || r > NBH) ? A_DS : ((H * NBH + r - 1 < NT) ? B_DS : 0);
+            return n;
+        }();
         // this row tile's share of the refill of the stage tile kt-1 used
-        constexpr int L0 = KS_I * LPS + (I * LPS) / MT, L1 = KS_I * LPS + ((I + 1) * LPS) / MT;
-        constexpr int LB = L0 < LOADS ? L0 : LOADS, LE = L1 < LOADS ? L1 : LOADS;
+        constexpr int P = KS_I * PH + H, NP = KS * PH;  // phase index inside the K tile
+        constexpr int PL0 = (P * LOADS) / NP, PL1 = ((P + 1) * LOADS) / NP;
+        constexpr int L0 = PL0 + (I * (PL1 - PL0)) / MH, L1 = PL0 + ((I + 1) * (PL1 - PL0)) / MH;
 #pragma unroll
-        for (int l = LB; l < LE; ++l) issue_one(refill, fill, l);
+        for (int l = L0; l < L1; ++l) issue_one(refill, fill, l);
         // Issue order: the LDS reads and direct loads of a row tile sit between its MFMAs.  All
         // waves leave the barrier together; if each first issued its loads and reads back to
         // back, they would queue at the CU's one memory pipeline while the matrix cores wait.
@@ -403,14 +420,26 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
         __builtin_amdgcn_sched_group_barrier(0x008, HEAD, 0);  // MFMA
         if constexpr (DS > 0) __builtin_amdgcn_sched_group_barrier(0x100, DS, 0);  // LDS reads
         if constexpr (NT - HEAD > 0) __builtin_amdgcn_sched_group_barrier(0x008, NT - HEAD, 0);
-        if constexpr (LE - LB > 0) __builtin_amdgcn_sched_group_barrier(0x020, LE - LB, 0);  // direct loads
+        if constexpr (L1 - L0 > 0) __builtin_amdgcn_sched_group_barrier(0x020, L1 - L0, 0);  // direct loads
     };
     auto kstep = [&](auto cur_c, auto ks_c) {
         constexpr int KS_I = decltype(ks_c)::value;
         constexpr bool last = (KS_I + 1 == KS);
         const int nstage = last ? next_stage : stage;
         constexpr int nks = last ? 0 : KS_I + 1;
-        static_for<MT>([&](auto i_c) { row_tile(cur_c, ks_c, i_c, nstage, nks); });
+        if constexpr (PH == 2) {
+            // phase 0 reads A for phase 1 of this k-step, phase 1 for phase 0 of the next one
+            static_for<MH>([&](auto i_c) {
+                row_tile(cur_c, ks_c, std::integral_constant<int, 0>{}, i_c, stage, KS_I, nstage, nks);
+            });
+            static_for<MH>([&](auto i_c) {
+                row_tile(cur_c, ks_c, std::integral_constant<int, 1>{}, i_c, nstage, nks, nstage, nks);
+            });
+        } else {
+            static_for<MH>([&](auto i_c) {
+                row_tile(cur_c, ks_c, std::integral_constant<int, 0>{}, i_c, nstage, nks, nstage, nks);
+            });
+        }
     };
     using std::integral_constant;
     if constexpr (KS == 1) {
@@ -442,20 +471,25 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
         // Ordering: every wave waits for its stores to be acknowledged before the workgroup
         // barrier, the arrival is counted after it, and the other half's partials are read only
         // by the workgroup that saw the count at one.
+        // 16-byte buffer stores and loads with the agent-scope bit (sc1): written through to
+        // memory and read past this XCD's L2, at full width (8-byte atomics write half lines).
         constexpr int PER_THREAD = MT * NT;  // f32x4 values
-        const int64_t tile_words = (int64_t)2 * kGemmThreads * PER_THREAD * 4;
-        float *mine = d.partial + (int64_t)task * tile_words + ((int64_t)half * kGemmThreads + tid) * PER_THREAD * 4;
-        float *theirs = d.partial + (int64_t)task * tile_words + ((int64_t)(half ^ 1) * kGemmThreads + tid) * PER_THREAD * 4;
+        constexpr int kAgentScope = 16;      // cache-policy bit sc1 of the buffer instructions
+        const int64_t tile_bytes = (int64_t)2 * kGemmThreads * PER_THREAD * 16;
+        char *tile_base = reinterpret_cast<char *>(d.partial) + (int64_t)task * tile_bytes;
+        const __amdgpu_buffer_rsrc_t rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(tile_base, 0, (int)tile_bytes, 0x00020000);
+        // [half][row tile * NT + column tile][thread]: a wave's store covers 1 KB in one piece
+        const int mine = (half * PER_THREAD * kGemmThreads + tid) * 16;
+        const int theirs = ((half ^ 1) * PER_THREAD * kGemmThreads + tid) * 16;
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
+        for (int i = 0; i < MT; ++i) {
 #pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                uint64_t w[2];
-                __builtin_memcpy(w, &acc[i][j], 16);
-                uint64_t *p = reinterpret_cast<uint64_t *>(mine + (i * NT + j) * 4);
-                __hip_atomic_store(p, w[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(p + 1, w[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            for (int j = 0; j < NT; ++j)
+                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rsrc,
+                                                       mine + (i * NT + j) * kGemmThreads * 16, 0, kAgentScope);
+            __builtin_amdgcn_sched_barrier(0);  // row tile by row tile: no pile of addresses and values
+        }
         drain_stores_then_barrier();
         lds_i32x *flag = (lds_i32x *)lds;
         if (tid == 0)
@@ -466,16 +500,15 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
         if (arrived_before == 0) return -1;
         if (tid == 0) __hip_atomic_store(d.arrivals + task, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-        for (int i = 0; i < MT; ++i)
+        for (int i = 0; i < MT; ++i) {
 #pragma unroll
             for (int j = 0; j < NT; ++j) {
-                const uint64_t *p = reinterpret_cast<const uint64_t *>(theirs + (i * NT + j) * 4);
-                uint64_t w[2] = {__hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
-                                 __hip_atomic_load(p + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)};
-                f32x4 o;
-                __builtin_memcpy(&o, w, 16);
-                acc[i][j] += o;
+                const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(
+                    rsrc, theirs + (i * NT + j) * kGemmThreads * 16, 0, kAgentScope);
+                acc[i][j] += __builtin_bit_cast(f32x4, w);
             }
+            __builtin_amdgcn_sched_barrier(0);  // a row tile's loads in flight at a time
+        }
     }
 
     // ---- epilogue: lane (m = lane%16, g = lane/16) holds C[m][4g .. 4g+3] of each 16x16 tile ----

@@ -1,24 +1,34 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path on one MI355X.  Prints ONE JSON line.
 
-Workload (BASELINE config 2): row-wise fp16 ops on X[16384,4096] ~ N(0,1) —
-reduce-sum over the last axis, softmax, RMSNorm (weight ~ U(0.5,1.5), eps 1e-6),
-fp32 accumulation — planned by the Planner and executed inside ONE persistent
-loop kernel (Model -> plan JSON -> Executor).  A "step" is one pass of the three
-ops over one X.  The plan holds four X tensors (4 x 128 MiB, plus separate
-outputs) and walks them in turn, so the 256 MB Infinity Cache cannot serve
-repeated reads; one plan iteration is therefore four steps.
+Headline (BASELINE config 2): row-wise fp16 ops on X[16384,4096] ~ N(0,1) — reduce-sum over
+the last axis, softmax, RMSNorm (weight ~ U(0.5,1.5), eps 1e-6), fp32 accumulation — planned
+by the Planner and executed inside ONE persistent loop kernel (Model -> plan JSON ->
+Executor).  The plan holds four X tensors (4 x 128 MiB, with outputs of their own) and walks
+them in turn, so the 256 MB Infinity Cache cannot serve repeated reads.  A "step" is one plan
+iteration: the three ops over each of the four X tensors (12 ops, 2.68 GB of algorithmic
+bytes).
 
-`value` is the whole-job throughput of the timed run of the resident loop kernel
-(host clock around run() + wait(), inputs already in HBM) in algorithmic GB/s.
-`roofline` prices the loop kernel itself against 8 TB/s: the same plan launched
-in one-shot mode (the kernel runs its iterations and returns) on torch's current
-stream, bracketed by HIP events, so one launch = `iterations` x 4 steps and its
-duration is what `rocprofv3 --kernel-trace` reports for that dispatch.  It also
-carries the same op bodies launched as three separate kernels, for comparison.
+`value` is the whole-job throughput of the timed run of the resident loop kernel (host clock
+around run() + wait(), inputs already in HBM) in algorithmic GB/s.  `roofline` prices the
+loop kernel itself against 8 TB/s: the same plan launched in one-shot mode (the kernel runs
+its iterations and returns) under HIP events on the stream it is launched on, which is the
+dispatch `rocprofv3 --kernel-trace` reports.
+
+`configs` holds the other BASELINE configurations (C1 GEMM, C3 SwiGLU FFN, C4 decode GEMV at
+batch 1 and 8, C5 decoder layer), each with the same kind of block: a HIP-event-timed one-shot
+launch of its loop kernel priced against its roofline, the resident loop kernel and the same
+ops as separate kernels beside it, and the CPU oracle timed on a bounded sample.  `machine`
+holds what this GPU sustains on an MFMA-only loop and on plain streams, beside the datasheet
+peaks used as denominators.
+
+Inputs come from the counter-based generator in ark_amd/prng.py (seed = hash of configuration
+and tensor name), drawn on the GPU; the CPU baseline reads the same rounded bits back.
 """
 import argparse
 import json
+import os
+import re
 import sys
 import time
 
@@ -32,17 +42,324 @@ ALGO_BYTES = {
 HBM_PEAK_GBPS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0
 NBUF = 4
+ROOT = os.path.dirname(os.path.abspath(__file__))
 
 
-# HBM bytes one step moves, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of the
-# one-shot loop-kernel dispatch (profiles/loop_kernel_rows_c2_pmc.txt: 387.50 MB
-# fetched + 268.51 MB written; counters scaled by a 128 MiB copy in the same run).
-MEASURED_TRAFFIC_BYTES_PER_STEP = 663834249
+def profiled_traffic_bytes_per_step():
+    """HBM bytes one step moves, as measured by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the
+    one-shot loop-kernel dispatch: read from the committed profile summary (not measured in
+    this run).  None when the summary is missing."""
+    path = os.path.join(ROOT, "profiles", "loop_kernel_rows_c2_pmc.txt")
+    try:
+        with open(path) as f:
+            m = re.search(r"^hbm_bytes_per_step:\s*(\d+)", f.read(), re.M)
+        return (int(m.group(1)), "profiles/loop_kernel_rows_c2_pmc.txt") if m else (None, None)
+    except OSError:
+        return None, None
 
 
-def cpu_baseline(x_np, w_np, min_seconds=8.0):
-    """The oracle (a port of the reference's host baselines) timed on this
-    machine's cores: whole-workload passes until `min_seconds` have gone by."""
+class Inputs:
+    """Seeded inputs drawn on the GPU, rounded once to the storage type."""
+
+    def __init__(self, torch, prng, config):
+        self.torch, self.prng, self.config = torch, prng, config
+
+    def normal(self, name, shape, dtype, std=1.0):
+        return self.prng.normal(self.prng.seed_of(self.config, name), tuple(shape), 0.0, std, device="cuda").to(dtype)
+
+    def uniform(self, name, shape, dtype, lo, hi):
+        return self.prng.uniform(self.prng.seed_of(self.config, name), tuple(shape), lo, hi, device="cuda").to(dtype)
+
+
+def _resident_us(torch, Executor, plan, iters, feeds):
+    """us per iteration in the resident loop kernel (host clock around run() + wait()):
+    `iters` untimed iterations (the clock settles over the first milliseconds of load), then
+    the median of three timed batches."""
+    ex = Executor(plan, device_id=0).compile()
+    for t, v in feeds:
+        ex.tensor_write_device(t, v)
+    torch.cuda.synchronize()
+    ex.launch()
+    ex.run(iters)
+    ex.wait()
+    batches = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        ex.run(iters)
+        ex.wait()
+        batches.append((time.perf_counter() - t0) / iters * 1e6)
+    info = ex.info()
+    ex.stop()
+    del ex
+    return sorted(batches)[1], info
+
+
+def _oneshot_and_separate_us(torch, Executor, plan, iters, feeds):
+    """(us per iteration of a one-shot launch of the loop kernel, us per iteration with every op
+    launched as a kernel of its own), both under HIP events on the executor's stream."""
+    side = torch.cuda.Stream()
+    ex = Executor(plan, device_id=0, stream=side.cuda_stream, loop_mode=False).compile()
+    for t, v in feeds:
+        ex.tensor_write_device(t, v)
+    torch.cuda.synchronize()
+    one, sep = [], []
+    with torch.cuda.stream(side):
+        ex.launch()
+        ex.run(iters)
+        ex.wait()
+        for _ in range(3):
+            s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s_.record()
+            ex.run(iters)
+            e_.record()
+            ex.wait()
+            torch.cuda.synchronize()
+            one.append(s_.elapsed_time(e_) / iters * 1e3)
+        ex.stop()
+        ex.run_separate(iters)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s_.record()
+            ex.run_separate(iters)
+            e_.record()
+            torch.cuda.synchronize()
+            sep.append(s_.elapsed_time(e_) / iters * 1e3)
+    del ex
+    return sorted(one)[1], sorted(sep)[1]
+
+
+def _block(workload, bound, work, one_us, loop_us, sep_us, info, cpu):
+    """One configuration's result: `work` is flop (bound mfma) or bytes (bound hbm) per iteration."""
+    if bound == "mfma":
+        achieved, peak, unit = work / one_us / 1e6, MFMA_PEAK_TFLOPS, "TFLOP/s"
+    else:
+        achieved, peak, unit = work / one_us / 1e3, HBM_PEAK_GBPS, "GB/s"
+    out = {"workload": workload,
+           "roofline": {"bound": bound, "kernel": f"arkmi_loop_kernel<{info['kernel_families']}> (one-shot launch)",
+                        "achieved": round(achieved, 1), "peak": peak, "unit": unit,
+                        "frac": round(achieved / peak, 4), "traffic": None,
+                        "us_per_iteration": round(one_us, 1)},
+           "resident_loop_kernel_us": round(loop_us, 1), "separate_kernels_us": round(sep_us, 1),
+           "loop_faster_than_separate": bool(loop_us < sep_us)}
+    if cpu is not None:
+        out["cpu_baseline"] = cpu
+    return out
+
+
+def _timed_cpu(fn, unit_work, unit, sample, min_seconds=2.0):
+    """Runs fn() until min_seconds have passed; work per call in `unit`-compatible quantity."""
+    from oracle import ark_oracle as O
+    fn()  # thread pool start-up outside the clock
+    n, t0 = 0, time.perf_counter()
+    while True:
+        fn()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= min_seconds:
+            break
+    return {"value": round(unit_work * n / dt / 1e9, 3), "unit": unit, "cores": O.num_threads(), "kind": "port",
+            "sample": f"{sample}; {n} passes in {dt:.1f} s"}
+
+
+def config_c1(torch, Model, Executor, inp, cpu):
+    a = inp.uniform("A", (4096, 4096), torch.float16, -1.0, 1.0)
+    b = inp.uniform("B", (4096, 4096), torch.float16, -1.0, 1.0)
+    m = Model()
+    ta, tb = m.tensor([4096, 4096], "fp16"), m.tensor([4096, 4096], "fp16")
+    m.matmul(ta, tb)
+    plan, feeds = m.plan(device_id=0), [(ta, a), (tb, b)]
+    loop_us, info = _resident_us(torch, Executor, plan, 20, feeds)
+    one_us, sep_us = _oneshot_and_separate_us(torch, Executor, plan, 20, feeds)
+    base = None
+    if cpu:
+        from oracle import ark_oracle as O
+        an, bn = a[:48].cpu().numpy(), b.cpu().numpy()
+        base = _timed_cpu(lambda: O.matmul(an, bn, "fp16"), 2.0 * 48 * 4096 * 4096, "GFLOP/s",
+                          "oracle matmul on 48 of the 4096 rows of A against all of B")
+    return _block("C1 fp16 GEMM C[4096,4096] = A . B, A, B ~ U[-1,1), fp32 accumulate", "mfma", 2.0 * 4096 ** 3,
+                  one_us, loop_us, sep_us, info, base)
+
+
+def config_c3(torch, Model, Executor, llama, inp, cpu):
+    fl = 3 * 2.0 * 8192 * 4096 * 11008
+    out = {}
+    for fused in (False, True):
+        m = Model()
+        tx = m.tensor([8192, 4096], "bf16")
+        ff = llama.FeedForward(m, 4096, 11008, "bf16")
+        ff.forward(tx, fused=fused)
+        vals = {"x": inp.normal("x", tx.shape, torch.bfloat16)}
+        feeds = [(tx, vals["x"])]
+        for name, t in ff.params().items():
+            vals[name] = inp.normal(name, t.shape, torch.bfloat16, 0.02)
+            feeds.append((t, vals[name]))
+        plan = m.plan(device_id=0)
+        loop_us, info = _resident_us(torch, Executor, plan, 10, feeds)
+        one_us, sep_us = _oneshot_and_separate_us(torch, Executor, plan, 10, feeds)
+        base = None
+        if cpu and fused:
+            from oracle import ark_oracle as O
+            xn = vals["x"][:16].view(torch.int16).cpu().numpy().view("uint16")
+            w1, w2, w3 = (vals[k].view(torch.int16).cpu().numpy().view("uint16") for k in ("w1", "w2", "w3"))
+
+            def ffn():
+                g = O.matmul(xn, w1, "bf16", trans_b=True)
+                u = O.matmul(xn, w3, "bf16", trans_b=True)
+                h = O.binary(O.binary(g, O.unary(g, "sigmoid", "bf16"), "mul", "bf16"), u, "mul", "bf16")
+                return O.matmul(h, w2, "bf16", trans_b=True)
+            base = _timed_cpu(ffn, 3 * 2.0 * 16 * 4096 * 11008, "GFLOP/s",
+                              "oracle FFN (reference composition) on 16 of the 8192 rows of x")
+        del feeds, vals
+        key = "fused_ops" if fused else "reference_composition"
+        out[key] = _block("C3 SwiGLU FFN x[8192,4096] bf16 -> 11008 -> 4096, one loop kernel ("
+                          + ("SwiGLU as one GEMM pass" if fused else "the reference's op-by-op composition") + ")",
+                          "mfma", fl, one_us, loop_us, sep_us, info, base)
+    return out
+
+
+def config_c4(torch, Model, Executor, inp, cpu):
+    shapes = [("W_qkv", 4096, 12288), ("W_o", 4096, 4096), ("W_gate_up", 4096, 22016), ("W_down", 11008, 4096)]
+    wbytes = float(sum(k * n * 2 for _, k, n in shapes))
+    out = {}
+    for bsz in (1, 8):
+        m = Model()
+        feeds, vals = [], []
+        for name, k, n in shapes:
+            tx, tw = m.tensor([bsz, k], "bf16"), m.tensor([k, n], "bf16")
+            m.matmul(tx, tw)
+            x, w = inp.normal(f"x_{name}_b{bsz}", tx.shape, torch.bfloat16), inp.normal(name, tw.shape, torch.bfloat16, 0.02)
+            feeds += [(tx, x), (tw, w)]
+            vals.append((x, w))
+        plan = m.plan(device_id=0)
+        loop_us, info = _resident_us(torch, Executor, plan, 50, feeds)
+        one_us, sep_us = _oneshot_and_separate_us(torch, Executor, plan, 50, feeds)
+        base = None
+        if cpu:
+            from oracle import ark_oracle as O
+            host = [(x.view(torch.int16).cpu().numpy().view("uint16"), w.view(torch.int16).cpu().numpy().view("uint16"))
+                    for x, w in vals]
+            base = _timed_cpu(lambda: [O.matmul(x, w, "bf16") for x, w in host], wbytes, "GB/s",
+                              f"oracle matmul of the whole step (four matrices, batch {bsz})")
+        del feeds, vals
+        out[f"batch{bsz}"] = _block(f"C4 decode GEMV, batch {bsz}: x[B,4096] . W_qkv[4096,12288], W_o[4096,4096], "
+                                    "W_gate/up[4096,22016], x[B,11008] . W_down[11008,4096], bf16, one plan",
+                                    "hbm", wbytes, one_us, loop_us, sep_us, info, base)
+    return out
+
+
+def config_c5(torch, np, Model, Executor, llama, inp, cpu):
+    names = {False: "reference_composition", True: "fused_ops", "attention": "fused_ops_attention_op"}
+    out = {}
+    for fused in (False, True, "attention"):
+        m = Model()
+        blk = llama.TransformerBlock(m, 4096, 32, 11008, "bf16")
+        tx = m.tensor([1, 2048, 4096], "bf16")
+        tf = m.tensor([1, 2048, 1, 128], "bf16")
+        tm = m.tensor([1, 1, 2048, 2048], "bf16")
+        blk.forward(tx, tf, tm, fused=bool(fused), causal=(fused == "attention"))
+        vals = {"x": inp.normal("hidden", tx.shape, torch.bfloat16)}
+        feeds = [(tx, vals["x"]),
+                 (tf, torch.from_numpy(llama.precompute_freqs_cis(128, 2048)).cuda().bfloat16()),
+                 (tm, torch.from_numpy(llama.causal_mask(2048, -np.inf)).cuda().bfloat16())]
+        if fused == "attention":
+            feeds.pop()  # the attention op applies the causal mask itself: no mask tensor in the plan
+        for name, t in blk.params().items():
+            vals[name] = (torch.ones(*t.shape, device="cuda") if name.endswith("_norm")
+                          else inp.normal(name, t.shape, torch.bfloat16, 0.02))
+            feeds.append((t, vals[name]))
+        plan = m.plan(device_id=0)
+        loop_us, info = _resident_us(torch, Executor, plan, 10, feeds)
+        one_us, sep_us = _oneshot_and_separate_us(torch, Executor, plan, 10, feeds)
+        # full (unskipped) attention counts 897.7 GFLOP; the attention op skips the masked key blocks
+        fl = 863.3e9 if fused == "attention" else 897.7e9
+        base = None
+        if cpu and fused == "attention":
+            from oracle import ark_oracle as O
+            host = {k: v.view(torch.int16).cpu().numpy().view("uint16") for k, v in vals.items() if v.dtype == torch.bfloat16}
+            xs = host["x"][0, :16]
+
+            def projections():
+                q = O.matmul(xs, host["attention.wq"], "bf16", trans_b=True)
+                o = O.matmul(q, host["attention.wo"], "bf16", trans_b=True)
+                g = O.matmul(o, host["feed_forward.w1"], "bf16", trans_b=True)
+                u = O.matmul(o, host["feed_forward.w3"], "bf16", trans_b=True)
+                h = O.binary(O.binary(g, O.unary(g, "sigmoid", "bf16"), "mul", "bf16"), u, "mul", "bf16")
+                return O.matmul(h, host["feed_forward.w2"], "bf16", trans_b=True)
+            base = _timed_cpu(projections, 2.0 * 16 * (2 * 4096 * 4096 + 3 * 4096 * 11008), "GFLOP/s",
+                              "oracle Q and output projections and the SwiGLU FFN on 16 of the 2048 positions "
+                              "(the K/V projections and the attention itself are left out of the CPU sample)")
+        del feeds, vals
+        out[names[fused]] = _block(
+            "C5 Llama-2-7B decoder layer, seq 2048, d 4096, 32 heads x 128, SwiGLU 11008, bf16, RoPE 10000, causal ("
+            + {False: "the reference's op-by-op composition", True: "fused ops, matmul/softmax attention",
+               "attention": "fused ops, attention as one op; flop count with masked key blocks skipped"}[fused] + ")",
+            "mfma", fl, one_us, loop_us, sep_us, info, base)
+    return out
+
+
+def machine_probes(torch, prng):
+    """What this GPU sustains: an MFMA-only loop (random and zero operands) and plain streams."""
+    import ctypes
+    from ark_amd._lib import lib, check
+    L = lib()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    sink = torch.zeros(16, device="cuda", dtype=torch.float32)
+    out = {"datasheet": {"mfma_dense_fp16_bf16_TFLOPs": MFMA_PEAK_TFLOPS, "hbm_GBps": HBM_PEAK_GBPS}}
+
+    def timed(fn, reps=5):
+        fn()
+        torch.cuda.synchronize()
+        s_, e_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s_.record()
+        for _ in range(reps):
+            fn()
+        e_.record()
+        torch.cuda.synchronize()
+        return s_.elapsed_time(e_) / reps * 1e-3
+
+    for label, data in (("random_U(-1,1)", prng.uniform(11, (1 << 20,), -1.0, 1.0, device="cuda").half()),
+                        ("zeros", torch.zeros(1 << 20, device="cuda", dtype=torch.float16))):
+        flops = ctypes.c_double()
+
+        def run():
+            check(L.arkmi_probe_mfma(ctypes.c_void_p(data.data_ptr()), ctypes.c_size_t(data.numel() * 2), ctypes.c_int(4000),
+                                     ctypes.c_void_p(sink.data_ptr()), ctypes.byref(flops), st))
+        sec = timed(run)
+        out[f"mfma_only_loop_TFLOPs_{label}"] = round(flops.value / sec / 1e12, 1)
+    nbytes = 1 << 28
+    src = torch.empty(nbytes, device="cuda", dtype=torch.uint8).random_()
+    dst = torch.empty_like(src)
+
+    def copy():
+        check(L.arkmi_probe_stream(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(dst.data_ptr()), ctypes.c_size_t(nbytes),
+                                   ctypes.c_void_p(sink.data_ptr()), st))
+
+    def read():
+        check(L.arkmi_probe_stream(ctypes.c_void_p(src.data_ptr()), ctypes.c_void_p(0), ctypes.c_size_t(nbytes),
+                                   ctypes.c_void_p(sink.data_ptr()), st))
+    out["stream_copy_GBps_read_plus_write"] = round(2 * nbytes / timed(copy, 10) / 1e9, 1)
+    out["stream_read_GBps"] = round(nbytes / timed(read, 10) / 1e9, 1)
+    return out
+
+
+def other_configs(torch, np, Model, Executor, llama, prng, cpu, only=None):
+    want = lambda c: only is None or only == c
+    out = {}
+    if want("c1"):
+        out["C1_gemm_fp16_4096"] = config_c1(torch, Model, Executor, Inputs(torch, prng, "C1"), cpu)
+    if want("c3"):
+        out["C3_ffn_bf16"] = config_c3(torch, Model, Executor, llama, Inputs(torch, prng, "C3"), cpu)
+    if want("c4"):
+        out["C4_decode_gemv_bf16"] = config_c4(torch, Model, Executor, Inputs(torch, prng, "C4"), cpu)
+    if want("c5"):
+        out["C5_llama7b_layer_seq2048_bf16"] = config_c5(torch, np, Model, Executor, llama, Inputs(torch, prng, "C5"), cpu)
+    return out
+
+
+def cpu_baseline_c2(x_np, w_np, min_seconds=8.0):
+    """The oracle (a port of the reference's host baselines) timed on this machine's cores:
+    passes over one X until `min_seconds` have gone by."""
     from oracle import ark_oracle as O
     O.lib()
     O.reduce(x_np[:256], -1, "sum", "fp16")  # thread pool start-up outside the clock
@@ -57,183 +374,20 @@ def cpu_baseline(x_np, w_np, min_seconds=8.0):
         if dt >= min_seconds:
             break
     total = sum(ALGO_BYTES.values()) * passes
-    return {"value": round(total / dt / 1e9, 3), "unit": "GB/s", "cores": O.num_threads(),
-            "kind": "port",
-            "sample": f"{passes} passes of the full step (reduce_sum+softmax+rmsnorm on "
-                      f"X[16384,4096] fp16) in {dt:.1f} s"}
-
-
-def _loop_vs_separate(torch, Executor, plan, iters, feeds=()):
-    """(us per iteration in the resident loop kernel, us per iteration with every op
-    launched as a kernel of its own) for one plan.  feeds: (tensor, torch tensor)
-    pairs written into both executors' arenas before the clock starts."""
-    # Both modes the same way: `iters` untimed iterations (the clock settles over the
-    # first few milliseconds of load), then three timed batches of `iters`, median.
-    ex = Executor(plan, device_id=0).compile()
-    for t, v in feeds:
-        ex.tensor_write_device(t, v)
-    torch.cuda.synchronize()
-    ex.launch()
-    ex.run(iters)
-    ex.wait()
-    batches = []
-    for _ in range(3):
-        t0 = time.perf_counter()
-        ex.run(iters)
-        ex.wait()
-        batches.append((time.perf_counter() - t0) / iters * 1e6)
-    loop_us = sorted(batches)[1]
-    ex.stop()
-    del ex
-    side = torch.cuda.Stream()
-    ex = Executor(plan, device_id=0, stream=side.cuda_stream, loop_mode=False).compile()
-    for t, v in feeds:
-        ex.tensor_write_device(t, v)
-    torch.cuda.synchronize()
-    batches = []
-    with torch.cuda.stream(side):
-        ex.run_separate(iters)
-        torch.cuda.synchronize()
-        for _ in range(3):
-            s_ = torch.cuda.Event(enable_timing=True)
-            e_ = torch.cuda.Event(enable_timing=True)
-            s_.record()
-            ex.run_separate(iters)
-            e_.record()
-            torch.cuda.synchronize()
-            batches.append(s_.elapsed_time(e_) / iters * 1e3)
-    sep_us = sorted(batches)[1]
-    del ex
-    return loop_us, sep_us
-
-
-def extra_configs(torch, ops, Model, Executor, g, kernel_us, only=None):
-    """Side measurements of the other BASELINE configurations (not the headline):
-    C1 GEMM, C3 SwiGLU FFN, C4 decode GEMV, C5 decoder layer, on seeded random
-    inputs of the stated distributions (operand values change the matrix cores'
-    power draw and with it the clock)."""
-    import numpy as np
-    from ark_amd import llama
-    extra = {}
-
-    def randn(shape, scale=1.0):
-        return (torch.randn(*shape, device="cuda", generator=g) * scale).bfloat16()
-
-    want = lambda c: only is None or only == c
-    if want("c1"):
-        _extra_c1(torch, ops, Model, Executor, g, kernel_us, extra)
-    if want("c3"):
-        _extra_c3(torch, Model, Executor, llama, randn, extra)
-    if want("c4"):
-        _extra_c4(torch, Model, Executor, randn, extra)
-    if want("c5"):
-        _extra_c5(torch, np, Model, Executor, llama, randn, extra)
-    return extra
-
-
-def _extra_c1(torch, ops, Model, Executor, g, kernel_us, extra):
-    # ---- C1: fp16 GEMM 4096^3 -------------------------------------------------------
-    a = (torch.rand(4096, 4096, device="cuda", generator=g) * 2 - 1).half()
-    b = (torch.rand(4096, 4096, device="cuda", generator=g) * 2 - 1).half()
-    c = torch.empty(4096, 4096, device="cuda", dtype=torch.float16)
-    fl = 2 * 4096 ** 3
-    us = kernel_us(lambda i: ops.matmul(a, b, out=c), reps=20)
-    extra["C1_gemm_fp16_4096_standalone"] = {"us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1),
-                                             "frac_of_2.5PF": round(fl / us / 1e6 / MFMA_PEAK_TFLOPS, 4)}
-    gm = Model()
-    ta, tb = gm.tensor([4096, 4096], "fp16"), gm.tensor([4096, 4096], "fp16")
-    gm.matmul(ta, tb)
-    gex = Executor(gm.plan(device_id=0), name="gemm").compile()
-    gex.tensor_write_device(ta, a)
-    gex.tensor_write_device(tb, b)
-    gex.launch()
-    gex.run(3)
-    gex.wait()
-    t0 = time.perf_counter()
-    gex.run(20)
-    gex.wait()
-    us = (time.perf_counter() - t0) / 20 * 1e6
-    gex.stop()
-    del gex
-    extra["C1_gemm_fp16_4096_in_loop_kernel"] = {"us": round(us, 1), "TFLOPs": round(fl / us / 1e6, 1),
-                                                 "frac_of_2.5PF": round(fl / us / 1e6 / MFMA_PEAK_TFLOPS, 4)}
-    del a, b, c
-
-
-def _extra_c3(torch, Model, Executor, llama, randn, extra):
-    # ---- C3: SwiGLU FFN x[8192,4096] bf16 -> 11008 -> 4096, one plan ----------------------
-    fl = 3 * 2 * 8192 * 4096 * 11008
-    for fused in (False, True):
-        m = Model()
-        tx = m.tensor([8192, 4096], "bf16")
-        ff = llama.FeedForward(m, 4096, 11008, "bf16")
-        ff.forward(tx, fused=fused)
-        feeds = [(tx, randn(tx.shape))] + [(t, randn(t.shape, 0.02)) for t in ff.params().values()]
-        loop_us, sep_us = _loop_vs_separate(torch, Executor, m.plan(device_id=0), 10, feeds)
-        del feeds
-        extra["C3_ffn_bf16_" + ("fused_ops" if fused else "reference_composition")] = {
-            "loop_kernel_us": round(loop_us, 1), "separate_kernels_us": round(sep_us, 1),
-            "loop_kernel_TFLOPs": round(fl / loop_us / 1e6, 1),
-            "frac_of_2.5PF": round(fl / loop_us / 1e6 / MFMA_PEAK_TFLOPS, 4)}
-
-
-def _extra_c4(torch, Model, Executor, randn, extra):
-    # ---- C4: decode GEMV, batch 1 and 8, the four Llama-2-7B weight shapes in one plan ---
-    shapes = [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]
-    wbytes = sum(k * n * 2 for k, n in shapes)
-    for bsz in (1, 8):
-        m = Model()
-        feeds = []
-        for (k, n) in shapes:
-            tx, tw = m.tensor([bsz, k], "bf16"), m.tensor([k, n], "bf16")
-            m.matmul(tx, tw)
-            feeds += [(tx, randn(tx.shape)), (tw, randn(tw.shape, 0.02))]
-        loop_us, sep_us = _loop_vs_separate(torch, Executor, m.plan(device_id=0), 50, feeds)
-        del feeds
-        extra[f"C4_decode_gemv_bf16_batch{bsz}"] = {
-            "loop_kernel_us": round(loop_us, 1), "separate_kernels_us": round(sep_us, 1),
-            "weight_bytes": wbytes, "loop_kernel_GBps": round(wbytes / loop_us / 1e3, 1),
-            "frac_of_8TBps": round(wbytes / loop_us / 1e3 / HBM_PEAK_GBPS, 4)}
-
-
-def _extra_c5(torch, np, Model, Executor, llama, randn, extra):
-    # ---- C5: one Llama-2-7B decoder layer, seq 2048, bf16 ------------------------------------
-    fl = 897.7e9  # full (unskipped) attention
-    names = {False: "reference_composition", True: "fused_ops", "attention": "fused_ops_attention_op"}
-    for fused in (False, True, "attention"):
-        m = Model()
-        blk = llama.TransformerBlock(m, 4096, 32, 11008, "bf16")
-        tx = m.tensor([1, 2048, 4096], "bf16")
-        tf = m.tensor([1, 2048, 1, 128], "bf16")
-        tm = m.tensor([1, 1, 2048, 2048], "bf16")
-        blk.forward(tx, tf, tm, fused=bool(fused), causal=(fused == "attention"))
-        feeds = [(tx, randn(tx.shape)),
-                 (tf, torch.from_numpy(llama.precompute_freqs_cis(128, 2048)).cuda().bfloat16()),
-                 (tm, torch.from_numpy(llama.causal_mask(2048, -np.inf)).cuda().bfloat16())]
-        if fused == "attention":
-            feeds.pop()  # the attention op applies the causal mask itself: no mask tensor in the plan
-        for name, t in blk.params().items():
-            feeds.append((t, torch.ones(*t.shape, device="cuda") if name.endswith("_norm")
-                          else randn(t.shape, 0.02)))
-        loop_us, sep_us = _loop_vs_separate(torch, Executor, m.plan(device_id=0), 10, feeds)
-        del feeds
-        extra["C5_llama7b_layer_seq2048_bf16_" + names[fused]] = {
-            "loop_kernel_us": round(loop_us, 1), "separate_kernels_us": round(sep_us, 1)}
-        if fused != "attention":  # the attention op skips the masked key blocks: fewer flops
-            extra["C5_llama7b_layer_seq2048_bf16_" + names[fused]]["loop_kernel_TFLOPs"] = \
-                round(fl / loop_us / 1e6, 1)
-
+    return {"value": round(total / dt / 1e9, 3), "unit": "GB/s", "cores": O.num_threads(), "kind": "port",
+            "sample": f"{passes} passes of reduce_sum+softmax+rmsnorm over one X[16384,4096] fp16 "
+                      f"(a quarter of a step) in {dt:.1f} s"}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=48)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--steps", type=int, default=12)
+    ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-extra", action="store_true", help="skip the side measurements (C1, C3, C4, C5)")
+    ap.add_argument("--no-extra", action="store_true", help="skip the other configurations (C1, C3, C4, C5)")
     ap.add_argument("--only", choices=["c1", "c3", "c4", "c5"], default=None,
-                    help="run only this side measurement and print it (for profiling one configuration)")
+                    help="run only this configuration and print its block (for profiling one configuration)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; this build has no multi-GPU path "
@@ -243,32 +397,20 @@ def main():
     import numpy as np
     import torch
     import ark_amd
-    from ark_amd import ops, Model, Executor
+    from ark_amd import Model, Executor, llama, prng
 
     torch.cuda.set_device(0)
     info = ark_amd.device_info(0)
-    g = torch.Generator(device="cuda").manual_seed(1234)
-
-    def kernel_us(fn, reps=40):
-        for i in range(4):
-            fn(i)
-        s = torch.cuda.Event(enable_timing=True)
-        e = torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        s.record()
-        for i in range(reps):
-            fn(i)
-        e.record()
-        torch.cuda.synchronize()
-        return s.elapsed_time(e) / reps * 1e3
+    cpu = not args.no_cpu_baseline
 
     if args.only:
         print(json.dumps({"only": args.only,
-                          "extra": extra_configs(torch, ops, Model, Executor, g, kernel_us, only=args.only)}))
+                          "configs": other_configs(torch, np, Model, Executor, llama, prng, cpu, only=args.only)}))
         return
 
-    xs = [torch.randn(ROWS, COLS, device="cuda", generator=g).half() for _ in range(NBUF)]
-    w = (torch.rand(COLS, device="cuda", generator=g) + 0.5).float()
+    inp = Inputs(torch, prng, "C2")
+    xs = [inp.normal(f"X{i}", (ROWS, COLS), torch.float16) for i in range(NBUF)]
+    w = inp.uniform("rmsnorm_weight", (COLS,), torch.float32, 0.5, 1.5)
 
     # ---- the workload as a model, planned and run in the loop kernel -------------
     m = Model()
@@ -284,24 +426,22 @@ def main():
     ex.tensor_write_device(tw, w)
     torch.cuda.synchronize()
 
-    steps = max(NBUF, (args.steps + NBUF - 1) // NBUF * NBUF)
-    warm = (args.warmup + NBUF - 1) // NBUF * NBUF
-    # The loop kernel stays resident between run() calls, so a device-wide
-    # synchronize inside the timed region would wait for it to leave;
-    # Executor.wait() is the completion point of a run.
+    steps, warm = max(1, args.steps), max(0, args.warmup)
+    # The loop kernel stays resident between run() calls, so a device-wide synchronize inside
+    # the timed region would wait for it to leave; Executor.wait() is the completion point.
     ex.launch()
     if warm:
-        ex.run(warm // NBUF)
+        ex.run(warm)
         ex.wait()
     t0 = time.perf_counter()
-    ex.run(steps // NBUF)
+    ex.run(steps)
     ex.wait()
     dt = time.perf_counter() - t0
     ex.stop()
     torch.cuda.synchronize()
     ms_per_step = dt / steps * 1e3
-    total_bytes = sum(ALGO_BYTES.values())
-    value = total_bytes / (ms_per_step * 1e-3) / 1e9
+    step_bytes = sum(ALGO_BYTES.values()) * NBUF
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     # spot check of the loop kernel's results on a few rows (full parity lives in tests/)
     got = torch.empty(ROWS, COLS, device="cuda", dtype=torch.float16)
@@ -312,88 +452,62 @@ def main():
     del ex
 
     # ---- roofline of the loop kernel: one-shot launches under HIP events ------------
-    # The executor launches on a torch stream (default priority), so torch's
-    # events, recorded on that stream, bracket the kernel.
+    # The executor launches on a torch stream (default priority), so torch's events, recorded
+    # on that stream, bracket the kernel.
     side = torch.cuda.Stream()
-    ex1 = Executor(plan, device_id=0, stream=side.cuda_stream, name="bench-oneshot",
-                   loop_mode=False).compile()
+    ex1 = Executor(plan, device_id=0, stream=side.cuda_stream, name="bench-oneshot", loop_mode=False).compile()
     for t, x in zip(tx, xs):
         ex1.tensor_write_device(t, x)
     ex1.tensor_write_device(tw, w)
     torch.cuda.synchronize()
-    iters = steps // NBUF
     launches = 10
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
-          for _ in range(launches)]
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
     with torch.cuda.stream(side):
         ex1.launch()
-        ex1.run(iters)
+        ex1.run(steps)
         ex1.wait()
         for s_, e_ in ev:
             s_.record()
-            ex1.run(iters)
+            ex1.run(steps)
             e_.record()
         ex1.wait()
     torch.cuda.synchronize()
     launch_ms = sum(s_.elapsed_time(e_) for s_, e_ in ev) / launches
     ex1.stop()
     del ex1
-    launch_bytes = total_bytes * steps
+    launch_bytes = step_bytes * steps
     achieved = launch_bytes / (launch_ms * 1e-3) / 1e9
 
-    # ---- the same op bodies as three separate kernels, HIP-event timed ---------------
-    douts = [torch.empty_like(xs[0]) for _ in range(NBUF)]
-    sums = torch.empty(ROWS, 1, device="cuda", dtype=torch.float16)
-    # a plain copy of known size (128 MiB read + 128 MiB written): the kernel the
-    # FETCH_SIZE / WRITE_SIZE counters of a --pmc run are scaled by
-    douts[0].copy_(xs[0])
-
-    per_kernel = {
-        "reduce_sum": kernel_us(lambda i: ops.reduce_sum(xs[i % NBUF], out=sums)),
-        "softmax": kernel_us(lambda i: ops.softmax(xs[i % NBUF], out=douts[i % NBUF])),
-        "rmsnorm": kernel_us(lambda i: ops.rmsnorm(xs[i % NBUF], w, eps=1e-6, out=douts[i % NBUF])),
-    }
-
-    def step_as_three_kernels(i):
-        x = xs[i % NBUF]
-        ops.reduce_sum(x, out=sums)
-        ops.softmax(x, out=douts[i % NBUF])
-        ops.rmsnorm(x, w, eps=1e-6, out=douts[(i + 1) % NBUF])
-
-    separate_us = kernel_us(step_as_three_kernels)
-    traffic = None
-    if MEASURED_TRAFFIC_BYTES_PER_STEP is not None:
-        traffic = MEASURED_TRAFFIC_BYTES_PER_STEP * steps
+    traffic_per_step, traffic_src = profiled_traffic_bytes_per_step()
     roofline = {"bound": "hbm",
-                "kernel": f"arkmi_loop_kernel<{kernel_families}> (one-shot launch of {iters} plan "
-                          f"iterations = {steps} steps)",
+                "kernel": f"arkmi_loop_kernel<{kernel_families}> (one-shot launch of {steps} plan iterations = steps)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "traffic": traffic_per_step * steps if traffic_per_step else None,
+                "traffic_source": (f"{traffic_src} (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE per step x steps; "
+                                   "not measured in this run)") if traffic_per_step else None,
                 "launch_ms": round(launch_ms, 4), "launch_algorithmic_bytes": launch_bytes,
-                "us_per_step_in_launch": round(launch_ms * 1e3 / steps, 2),
-                "separate_kernels_us_per_step": round(separate_us, 2),
-                "separate_kernel_us": {k: round(v, 2) for k, v in per_kernel.items()},
-                "separate_kernel_GBps": {k: round(ALGO_BYTES[k] / (v * 1e-6) / 1e9, 1)
-                                         for k, v in per_kernel.items()}}
+                "us_per_step_in_launch": round(launch_ms * 1e3 / steps, 2)}
 
     out = {
-        "metric": "GEMV/reduce HBM GB/s vs roofline (row ops reduce_sum+softmax+rmsnorm in one loop kernel)",
+        "metric": "GEMV/reduce HBM GB/s vs roofline (row ops reduce_sum+softmax+rmsnorm in one loop kernel; "
+                  "algorithmic bytes per second through L2 and fabric: the three ops of an X re-read the same "
+                  "128 MiB, which the Infinity Cache may serve)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps,
         "warmup": warm, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": "C2 row ops: X[16384,4096] fp16 ~N(0,1), reduce_sum + softmax + "
                                "RMSNorm(w~U(0.5,1.5), eps=1e-6), fp32 accumulate, one persistent loop "
-                               "kernel, 4 rotating X tensors",
+                               "kernel; a step = the three ops over each of 4 rotating X tensors",
                    "device": info["gcn_arch"], "num_cu": info["num_cu"]},
         "roofline": roofline,
+        "machine": machine_probes(torch, prng),
     }
-
     if not args.no_extra:
-        out["extra"] = extra_configs(torch, ops, Model, Executor, g, kernel_us)
-
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(xs[0].cpu().numpy(), w.cpu().numpy())
+        out["configs"] = other_configs(torch, np, Model, Executor, llama, prng, cpu)
+    if cpu:
+        out["cpu_baseline"] = cpu_baseline_c2(xs[0].cpu().numpy(), w.cpu().numpy())
     print(json.dumps(out))
 
 

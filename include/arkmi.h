@@ -137,6 +137,17 @@ int arkmi_gemv_static(int dtype, const void *x, const void *w, void *y, int m, i
                       int k, int64_t ldx, int64_t ldw, int64_t ldy, int num_tasks,
                       void *stream);
 
+/* Measurement probes (no counterpart in the reference): what this machine sustains, to print
+ * beside the datasheet peaks.  Each call launches one kernel on `stream`; the caller times it.
+ *   arkmi_probe_mfma: every CU's 8 waves run `iters` rounds of 16 independent
+ *     v_mfma_f32_16x16x32_f16 on operands read from `operands` (>= 1 MiB; random values draw more
+ *     power than zeros and lower the clock); *flops receives the flops of the launch.
+ *   arkmi_probe_stream: reads `bytes` from src with 16-byte loads and writes them to dst (a copy)
+ *     or, with dst == NULL, only reads.  `sink` is 4 bytes of device memory the kernels may write. */
+int arkmi_probe_mfma(const void *operands, size_t operand_bytes, int iters, void *sink,
+                     double *flops, void *stream);
+int arkmi_probe_stream(const void *src, void *dst, size_t bytes, void *sink, void *stream);
+
 /* ------------------------------------------------------------------------
  * Model building and planning for bindings that cannot use the C++ classes
  * directly.  Every call maps onto one member of ark::Model / PlannerContext /

@@ -7,13 +7,14 @@ TORCH_DT = {"fp32": torch.float32, "fp16": torch.float16, "bf16": torch.bfloat16
 
 
 def make(oracle, shape, dtype, seed, dist="normal", lo=-1.0, hi=1.0, scale=1.0):
-    """Seeded values rounded once to the storage dtype; CPU oracle and GPU read
-    the same bits.  Returns the numpy storage array."""
-    rng = np.random.default_rng(seed)
+    """Seeded values from the counter-based generator the benchmark draws from too
+    (ark_amd/prng.py), rounded once to the storage dtype; CPU oracle and GPU read the
+    same bits.  Returns the numpy storage array."""
+    from ark_amd import prng
     if dist == "normal":
-        x = rng.standard_normal(shape, dtype=np.float32) * scale
+        x = prng.normal(seed, tuple(shape), 0.0, scale)
     else:
-        x = rng.uniform(lo, hi, size=shape).astype(np.float32)
+        x = prng.uniform(seed, tuple(shape), lo, hi)
     return oracle.to_storage(x, dtype)
 
 

@@ -864,7 +864,7 @@ def test_matmul_split_k(oracle, dtype, trans_other):
     sampled rows against the oracle, and bit for bit against the same plan run one kernel per op."""
     import torch
     from ark_amd import Model, Executor
-    M, N, K = 2048, 4096, 2048
+    M, N, K = 2048, 4096, 8192
     a = make(oracle, (M, K), dtype, 111, "uniform")
     b = make(oracle, (N, K) if trans_other else (K, N), dtype, 112, "normal", scale=0.05)
     m = Model()
@@ -891,7 +891,7 @@ def test_matmul_split_k_with_follower_and_neighbours(oracle):
     ops before and after it keep their grid barriers (a split tile has no fixed workgroup)."""
     from ark_amd import Model
     dtype = "bf16"
-    M, N, K = 2048, 4096, 2048
+    M, N, K = 2048, 4096, 8192
     x = make(oracle, (M, K), dtype, 113, "normal")
     w = make(oracle, (N, K), dtype, 114, "normal", scale=0.02)
     r = make(oracle, (M, N), dtype, 115, "normal")

@@ -349,8 +349,8 @@ def test_rocm950_matmul_tile_choice():
         c = json.loads(m.plan(arch="ROCM_950", num_processors=256))["TaskInfos"][0]["Ops"][0]["Config"]
         return c["TileShapeMNK"][:2], c["NumTasks"]
     assert tile(8192, 11008, 4096) == ([256, 256], 32 * 43)
-    assert tile(2048, 4096, 4096) == ([256, 256], 2 * 8 * 16)     # 128 large tiles, K split in two
-    assert tile(2048, 4096, 1024) == ([128, 256], 16 * 16)        # short K: smaller tiles instead
+    assert tile(2048, 4096, 4096) == ([128, 256], 16 * 16)        # 256x256 would leave CUs idle
+    assert tile(2048, 4096, 11008 // 128 * 128) == ([256, 256], 2 * 8 * 16)  # long K: large tiles, K split in two
     assert tile(2048, 2048, 128, batch=(1, 32)) == ([256, 256], 32 * 64)
     assert tile(512, 512, 64) == ([128, 128], 16)
     with pytest.raises(ArkmiError) as e:
@@ -395,13 +395,13 @@ def test_rocm950_matmul_tiles_and_split_k():
         return json.loads(m.plan(arch="ROCM_950", num_processors=ncu))["TaskInfos"][0]["Ops"][0]["Config"]
     c = cfg(4096, 4096, 4096)
     assert c["TileShapeMNK"][:2] == [256, 256] and c["NumTasks"] == 256 and "SplitK" not in c
-    c = cfg(2048, 4096, 4096, trans_other=True)
+    c = cfg(2048, 4096, 8192, trans_other=True)
     assert c["TileShapeMNK"][:2] == [256, 256] and c["SplitK"] == 2 and c["NumTasks"] == 256
     c = cfg(2048, 4096, 11008, trans_other=True)
     assert c["SplitK"] == 2 and c["NumTasks"] == 256
-    c = cfg(2048, 4096, 1024)                       # short K: not worth splitting
-    assert "SplitK" not in c and c["NumTasks"] >= 256
+    c = cfg(2048, 4096, 4096)                       # the exchange of partial sums would cost what the tile gains
+    assert "SplitK" not in c and c["TileShapeMNK"][:2] == [128, 256] and c["NumTasks"] == 256
     c = cfg(2048, 2048, 4096)                       # 64 large tiles: smaller tiles fill the chip instead
     assert "SplitK" not in c and c["TileShapeMNK"][:2] == [128, 128]
-    c = cfg(2048, 4096, 4096, ncu=128)              # a plan for 128 processors has a tile for each already
+    c = cfg(2048, 4096, 8192, ncu=128)              # a plan for 128 processors has a tile for each already
     assert "SplitK" not in c and c["TileShapeMNK"][:2] == [256, 256] and c["NumTasks"] == 128
