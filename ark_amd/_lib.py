@@ -15,13 +15,39 @@ _STATUS_NAMES = {1: "InternalError", 2: "InvalidUsageError", 3: "ModelError",
 
 
 class ArkmiError(RuntimeError):
-    """A non-zero status from the C ABI; `.code` is the arkmi_status value and
-    `.kind` the name of the matching ark:: error class."""
+    """Base of the error classes (ark::BaseError, ark/include/ark/error.hpp:13-43).
+    Raised by check() for a non-zero status from the C ABI: `.code` is the
+    arkmi_status value and `.kind` the name of the matching ark:: error class,
+    and the object is an instance of the subclass of that name.  Raised from
+    Python with a message alone, str() is that message."""
+    code = 0
 
-    def __init__(self, code, msg):
-        self.code = code
-        self.kind = _STATUS_NAMES.get(code, "Error")
-        super().__init__(f"{self.kind}: {msg}")
+    def __init__(self, *args):
+        if len(args) == 2 and isinstance(args[0], int):
+            self.code = args[0]
+            self.kind = _STATUS_NAMES.get(args[0], "Error")
+            super().__init__(f"{self.kind}: {args[1]}")
+        else:
+            self.kind = _STATUS_NAMES.get(self.code, "Error")
+            super().__init__(*args)
+
+
+BaseError = ArkmiError
+
+
+def _error_class(code, name):
+    return type(name, (ArkmiError,), {"code": code, "__doc__": f"ark::{name}"})
+
+
+InternalError = _error_class(1, "InternalError")
+InvalidUsageError = _error_class(2, "InvalidUsageError")
+ModelError = _error_class(3, "ModelError")
+PlanError = _error_class(4, "PlanError")
+UnsupportedError = _error_class(5, "UnsupportedError")
+SystemError = _error_class(6, "SystemError")  # noqa: A001 (the reference's name)
+GpuError = _error_class(7, "GpuError")
+_ERROR_CLASSES = {c.code: c for c in (InternalError, InvalidUsageError, ModelError, PlanError,
+                                      UnsupportedError, SystemError, GpuError)}
 
 
 class DeviceInfo(ctypes.Structure):
@@ -52,7 +78,8 @@ def lib():
 
 def check(status):
     if status != 0:
-        raise ArkmiError(status, lib().arkmi_last_error().decode(errors="replace"))
+        raise _ERROR_CLASSES.get(status, ArkmiError)(
+            status, lib().arkmi_last_error().decode(errors="replace"))
 
 
 def device_info(device_id=0):

@@ -1052,6 +1052,7 @@ struct Executor {
                 g.task_b = st.task_b; g.task_e = st.task_e; g.task_s = st.task_s; g.gran = st.gran;
                 g.n_slots = st.n_slots; g.slot_warps = st.slot_warps; g.slot_sram = st.slot_sram;
                 g.op_begin = (int)ops.size();
+                g.signal_begin = -1;
                 const Json &ti = task_infos.at((size_t)st.task_info);
                 const Json &ops_json = ti.at("Ops");
                 if (ops_json.size() > 1 && (st.n_slots != 1 || st.slot_warps != block_warps))
@@ -1075,6 +1076,23 @@ struct Executor {
                 for (const auto &oj : ops_json.elements())
                     ops.push_back(lower_op(oj, L, st.slot_warps, block_warps, st.n_slots, st.slot_sram));
                 g.op_count = (int)ops.size() - g.op_begin;
+                // the loop kernel runs one task loop per kind of the first op; behind a matmul
+                // come elementwise ops only, behind a small op any small op
+                if (g.op_count > 1) {
+                    const int k0 = ops[(size_t)g.op_begin].kind;
+                    if (k0 == DEV_GEMV || k0 == DEV_ATTN)
+                        ARK_ERR(UnsupportedError, "task ", st.task_info, ": no op can be fused behind a skinny matmul or "
+                                "an attention op");
+                    for (int o = g.op_begin + 1; o < (int)ops.size(); ++o) {
+                        const int ko = ops[(size_t)o].kind;
+                        if (ko == DEV_GEMM || ko == DEV_GEMV || ko == DEV_ATTN)
+                            ARK_ERR(UnsupportedError, "task ", st.task_info, ": a matmul or attention op must be the "
+                                    "first op of its task");
+                        if (k0 == DEV_GEMM && ko != DEV_EWISE)
+                            ARK_ERR(UnsupportedError, "task ", st.task_info, ": only elementwise ops can be fused "
+                                    "behind a matmul");
+                    }
+                }
                 int group_fam = 0;
                 for (int o = g.op_begin; o < (int)ops.size(); ++o)
                     group_fam |= ops[o].kind == DEV_ROW ? (ops[o].row.red_len > 0 ? FAM_EXT : FAM_ROW)

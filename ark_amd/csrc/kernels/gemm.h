@@ -335,7 +335,6 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     //
     static_assert(S >= 3, "the ring needs the current, the next and one tile in flight");
     const int KT = k_len / BK;
-    constexpr int LPS = (LOADS + KS - 1) / KS;  // direct loads issued per k-step
     constexpr int B_DS = TRANS_B ? 1 : 2, A_DS = TRANS_A ? 2 : 1;  // LDS reads per fragment
 
     s.sync();  // the previous task is done with the stage buffers

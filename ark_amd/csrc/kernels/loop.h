@@ -54,8 +54,24 @@ struct DevTaskGroup {
     int32_t n_slots, slot_warps, slot_sram;
     int32_t op_begin, op_count;
     int32_t trace_offset;  // first trace record of this group, -1 if not traced
-    int32_t pad_[2];
+    // Dependency counters (the fields are dead when LoopProgram::dep_counters is null).
+    // As a consumer: before task index i runs, the counters [lo, hi] of each of the group's
+    // n_waits producers must have reached expect * iteration; (lo, hi) of wait w are the words
+    // wait_spans[span_begin + 2 * (i * n_waits + w)] and the next one.
+    int32_t n_waits, wait_begin, span_begin;
+    // As a producer: task index i completes row block signal_map[signal_begin + i] and adds one
+    // to counter signal_base + that block; signal_begin < 0: the group signals nothing.
+    int32_t signal_begin, signal_base;
+    int32_t pad_[1];
 };
+
+// One producer a task group waits for.
+struct DevWait {
+    int32_t counter_base;  // first counter of the producer's row blocks
+    int32_t expect;        // tasks per row block, i.e. what one iteration adds to each counter
+};
+
+constexpr int kDepStride = 16;  // words between two dependency counters: one per 64-byte line
 
 // STEP_LOCAL_SYNC: the next group depends only on what this workgroup itself wrote
 enum DevStepKind : int32_t { STEP_BARRIER = 0, STEP_TASKS = 1, STEP_LOCAL_SYNC = 2 };
@@ -107,12 +123,33 @@ struct LoopProgram {
     // each step of the last iteration, plus one entry for the end of the body
     // ([num_blocks][num_steps + 1])
     unsigned long long *step_clock;
+    // Dependency counters in place of some grid barriers; all four null when the plan has none
+    // (and in the one-op kernels, where kernel boundaries order everything).  The counters are
+    // zeroed before every launch and only grow.
+    const DevWait *waits;
+    const int32_t *wait_spans;
+    const int32_t *signal_map;
+    unsigned int *dep_counters;
     int32_t num_steps;
     int32_t num_blocks;
     // what separates two iterations of the body inside one command:
     // 2 a grid barrier, 1 a workgroup-local sync, 0 nothing
     int32_t iter_sync;
     int32_t pad_;
+};
+
+struct HostMailbox;
+
+// The one kernel parameter of the loop kernel and of the one-op kernels.  The kernels read it
+// through the kernel-argument segment whenever a field is needed instead of keeping the fields
+// in registers across the op bodies.
+struct LoopArgs {
+    LoopProgram prog;
+    LoopControl *ctl;
+    HostMailbox *mb;
+    uint64_t idle_ticks, wait_ticks;
+    int32_t one_shot_iters;  // loop kernel: > 0 runs that many iterations and returns
+    int32_t group;           // one-op kernel: the task group to run
 };
 
 // Mapped, pinned host memory shared with the kernel.

@@ -50,8 +50,12 @@ const void *step_kernel_select(int families) {
 
 void step_kernel_launch(const void *kernel, const LoopProgram &prog, int group, int grid, int threads,
                         int lds_bytes, hipStream_t stream) {
-    LoopProgram p = prog;
-    void *args[] = {&p, &group};
+    LoopArgs a{};
+    a.prog = prog;
+    // kernel boundaries order the ops: no dependency counters
+    a.prog.waits = nullptr; a.prog.wait_spans = nullptr; a.prog.signal_map = nullptr; a.prog.dep_counters = nullptr;
+    a.group = group;
+    void *args[] = {&a};
     ARKMI_HIP(hipLaunchKernel(kernel, dim3(grid), dim3(threads), args, (size_t)lds_bytes, stream));
 }
 
@@ -91,8 +95,12 @@ void loop_kernel_launch(const void *kernel, const LoopProgram &prog, LoopControl
                         HostMailbox *mb_dev, int grid, int threads, int lds_bytes,
                         int one_shot_iters, uint64_t idle_ticks, uint64_t wait_ticks,
                         hipStream_t stream) {
-    LoopProgram p = prog;
-    void *args[] = {&p, &ctl, &mb_dev, &one_shot_iters, &idle_ticks, &wait_ticks};
+    LoopArgs a{};
+    a.prog = prog;
+    a.ctl = ctl; a.mb = mb_dev;
+    a.idle_ticks = idle_ticks; a.wait_ticks = wait_ticks;
+    a.one_shot_iters = one_shot_iters;
+    void *args[] = {&a};
     ARKMI_HIP(hipLaunchKernel(kernel, dim3(grid), dim3(threads), args, (size_t)lds_bytes, stream));
 }
 

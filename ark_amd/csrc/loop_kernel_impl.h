@@ -27,7 +27,7 @@ __device__ __forceinline__ bool in_range(int x, int b, int e, int s) {
 // Sense-free counting barrier over `nblocks` workgroups.  Agent-scope release /
 // acquire fences order the blocks' global writes across the XCDs' L2s.
 // Returns false (uniformly per block) once `abort` has been raised.
-static __device__ bool grid_barrier(GridBarrier *bar, unsigned nblocks, LoopControl *ctl,
+__device__ __forceinline__ bool grid_barrier(GridBarrier *bar, unsigned nblocks, LoopControl *ctl,
                              uint64_t limit_ticks) {
     int *lds_flag = reinterpret_cast<int *>(g_loop_lds);
     // every wave's stores are acknowledged by the L2 before thread 0 writes the L2 back
@@ -94,7 +94,7 @@ __device__ __forceinline__ unsigned xcc_id() {
 // Polls *word until it has reached `target` (counters only grow; the comparison
 // is safe across 32-bit wrap-around); false once `abort` is raised or the time
 // limit has passed (then `abort` is raised for everyone).
-static __device__ bool poll_reached(unsigned *word, unsigned target, LoopControl *ctl, uint64_t limit_ticks) {
+__device__ __forceinline__ bool poll_reached(unsigned *word, unsigned target, LoopControl *ctl, uint64_t limit_ticks) {
     const uint64_t t0 = wall_clock64();
     unsigned polls = 0;
     // relaxed polls: an acquire load would invalidate this XCD's L2 on every
@@ -117,7 +117,7 @@ static __device__ bool poll_reached(unsigned *word, unsigned target, LoopControl
 // when its counter reaches e * nx, and on the chip when the top counter
 // reaches e * nxcd, so an arrival is one atomic and nothing is ever reset.
 // Returns false (uniformly per block) once `abort` has been raised.
-static __device__ bool grid_barrier_xcd(LoopControl *ctl, XcdInfo &xi, uint64_t limit_ticks) {
+__device__ __forceinline__ bool grid_barrier_xcd(LoopControl *ctl, XcdInfo &xi, uint64_t limit_ticks) {
     int *lds_flag = reinterpret_cast<int *>(g_loop_lds);
     xi.epoch += 1u;
     // every wave waits until the L2 has acknowledged its stores, then the workgroup
@@ -136,7 +136,9 @@ static __device__ bool grid_barrier_xcd(LoopControl *ctl, XcdInfo &xi, uint64_t 
             __hip_atomic_store(&xb->generation, xi.epoch, __ATOMIC_RELAXED, AGENT);
         } else {
             poll_reached(&xb->generation, xi.epoch, ctl, limit_ticks);
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // this CU's L1
+            // This CU's L1 only: the XCD's L2 has just been invalidated by its last arriver,
+            // and an agent-scope acquire here would walk that L2 once more per workgroup.
+            asm volatile("buffer_inv sc0" ::: "memory");
         }
         *lds_flag = __hip_atomic_load(&ctl->abort, __ATOMIC_RELAXED, AGENT) ? 0 : 1;
     }
@@ -164,223 +166,427 @@ __device__ __forceinline__ D load_const(const D *p) {
     return d;
 }
 
-// Returns the task index the ops fused behind the matmul run for (the tile this workgroup
-// finished), -1 when another workgroup finishes the tile (a split of K).
+// FAM is the set of op families compiled into this kernel variant.  A plan runs on the
+// smallest variant that holds its families.
+//
+// The long-running bodies (matmul tiles, skinny matmul, attention) are functions of their own,
+// not inlined into the kernel: each gets its own register allocation and instruction schedule,
+// the same in every variant, in the loop kernel and in the one-op kernels alike.  (Inlined, the
+// K loop of a matmul tile came out differently depending on what surrounded it: in the loop
+// kernel its loads were issued later and it carried five more waits than in a kernel of its
+// own, and ran 10-15 % slower.)  Arguments of a device function arrive in vector registers, so
+// a body takes only indices and reads everything uniform itself: its descriptor from the op
+// table (through the kernel arguments), into scalar registers.
+
+// The small bodies (elementwise ops, row ops, the embedding gather) for one task, inlined.
+template <int FAM>
+__device__ __forceinline__ void run_small(const DevOp *op, int task, const Slot &s) {
+    const int kind = load_const(&op->kind);
+    if (kind == DEV_EWISE) {
+        if constexpr ((FAM & FAM_EWISE) != 0) {
+            const EwiseDesc d = load_const(&op->ew);
+            ewise_dispatch(d, task, s);
+        }
+    } else if (kind == DEV_ROW) {
+        if (load_const(&op->row.red_len) > 0) {
+            if constexpr ((FAM & FAM_EXT) != 0) {
+                const RowOpDesc d = load_const(&op->row);
+                reduce_axis_dispatch(d, task, s);
+            }
+        } else if constexpr ((FAM & FAM_ROW) != 0) {
+            const RowOpDesc d = load_const(&op->row);
+            row_op_dispatch(d, task, s);
+        }
+    } else if (kind == DEV_EMBED) {
+        if constexpr ((FAM & FAM_EXT) != 0) {
+            const EmbedDesc d = load_const(&op->emb);
+            embedding_task(d, task, s);
+        }
+    }
+}
+
+// An elementwise op fused behind a matmul in the same task (the host admits no other kind
+// there).  The thread index is made opaque per task: the per-lane addresses the body derives
+// from it would otherwise be lifted out of the task loop and stay in registers across the matmul.
+template <int FAM>
+__device__ __forceinline__ void run_follower(const DevOp *op, int task, const Slot &s_in) {
+    if constexpr ((FAM & FAM_EWISE) != 0) {
+        Slot s = s_in;
+        asm volatile("" : "+v"(s.tid));
+        const EwiseDesc d = load_const(&op->ew);
+        ewise_dispatch(d, task, s);
+    }
+}
+
+// The kernel's one parameter, read where a field is needed: the pointer to the kernel-argument
+// segment is made opaque on every access, so no load from it is shared with an earlier one or
+// lifted out of a loop, and no field occupies a scalar register across an op body (a matmul
+// body needs nearly all of them; with the loop's own state resident beside it the K loop came
+// out with later loads and more waits than the same body in a kernel of its own).
+__device__ __forceinline__ const ARKMI_CONST LoopArgs *kargs() {
+    const ARKMI_CONST LoopArgs *p = (const ARKMI_CONST LoopArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));
+    return p;
+}
+
+template <typename D>
+__device__ __forceinline__ D load_karg(const ARKMI_CONST D *p) {
+    static_assert(sizeof(D) % 4 == 0, "kernel-argument fields are whole words");
+    D d;
+    uint32_t w[sizeof(D) / 4];
+    const ARKMI_CONST uint32_t *src = (const ARKMI_CONST uint32_t *)p;
+#pragma unroll
+    for (size_t i = 0; i < sizeof(D) / 4; ++i) w[i] = src[i];
+    __builtin_memcpy(&d, w, sizeof(D));
+    return d;
+}
+#define KARG(field) load_karg(&kargs()->field)
+
+// ---- the long-running bodies -----------------------------------------------------------------
+#define ARKMI_BODY __device__ __attribute__((noinline))
+
+// A long-running op owns the whole workgroup (checked on the host): its slot is the first one.
+__device__ __forceinline__ Slot body_slot(int tid) {
+    Slot s;
+    s.tid = tid;
+    s.nthreads = blockDim.x;
+    s.lds = (lds_ptr)g_loop_lds + kLdsReserved;
+    s.lds_bytes = 0;
+    s.whole_block = true;
+    return s;
+}
+
+__device__ __forceinline__ const DevOp *body_op(int op_index) {
+    return KARG(prog.ops) + __builtin_amdgcn_readfirstlane(op_index);
+}
+
+// One matmul tile shape.  Returns the task index the ops fused behind the matmul run for (the
+// tile this workgroup finished), -1 when another workgroup finishes the tile (a split of K).
+template <typename T, int BM, int BN, bool TRANS_B, bool TRANS_A = false, bool DUAL_B = false, bool SPLIT = false>
+ARKMI_BODY int gemm_body(int op_index, int task, int tid) {
+    const GemmDesc g = load_const(&body_op(op_index)->gemm);
+    return gemm_tile<T, BM, BN, TRANS_B, EpilogueStore, TRANS_A, DUAL_B, SPLIT>(
+        g, __builtin_amdgcn_readfirstlane(task), body_slot(tid), EpilogueStore());
+}
+
+ARKMI_BODY int gemm_f32_body(int op_index, int task, int tid) {
+    const GemmDesc g = load_const(&body_op(op_index)->gemm);
+    gemm_f32_dispatch(g, __builtin_amdgcn_readfirstlane(task), body_slot(tid));
+    return task;
+}
+
+ARKMI_BODY int gemv_body(int op_index, int task, int tid) {
+    const GemvDesc d = load_const(&body_op(op_index)->gemv);
+    gemv_dispatch(d, __builtin_amdgcn_readfirstlane(task), body_slot(tid));
+    return task;
+}
+
+ARKMI_BODY int attn_body(int op_index, int task, int tid) {
+    const AttnDesc d = load_const(&body_op(op_index)->attn);
+    attn_dispatch(d, __builtin_amdgcn_readfirstlane(task), body_slot(tid));
+    return task;
+}
+
 template <int FAM, typename T, bool TRANS_B>
-__device__ __forceinline__ int gemm_by_tile(const DevOp *op, int task, const Slot &s) {
-    const GemmDesc g = load_const(&op->gemm);
+__device__ __forceinline__ int gemm_by_tile(const DevOp *op, int op_index, int task, int tid) {
     const int tm = load_const(&op->gemm_tile_m), tn = load_const(&op->gemm_tile_n);
-    if (g.split_k == 2) {  // 256x256 tiles only (checked on the host)
+    if (load_const(&op->gemm.split_k) == 2) {  // 256x256 tiles only (checked on the host)
         if constexpr ((FAM & FAM_SPLITK) != 0)
-            return gemm_tile<T, 256, 256, TRANS_B, EpilogueStore, false, false, true>(g, task, s, EpilogueStore());
+            return gemm_body<T, 256, 256, TRANS_B, false, false, true>(op_index, task, tid);
         else
             return -1;
     }
     if constexpr (TRANS_B) {
-        if (g.b2) {  // gate/up pair: 256-wide tiles only (checked on the host)
-            if (tm == 256) return gemm_tile<T, 256, 256, true, EpilogueStore, false, true>(g, task, s, EpilogueStore());
-            return gemm_tile<T, 128, 256, true, EpilogueStore, false, true>(g, task, s, EpilogueStore());
+        if (load_const(&op->gemm.b2) != nullptr) {  // gate/up pair: 256-wide tiles only (checked on the host)
+            if (tm == 256) return gemm_body<T, 256, 256, true, false, true>(op_index, task, tid);
+            return gemm_body<T, 128, 256, true, false, true>(op_index, task, tid);
         }
     }
-    if (tm == 256 && tn == 256) return gemm_tile<T, 256, 256, TRANS_B>(g, task, s, EpilogueStore());
-    if (tm == 128 && tn == 256) return gemm_tile<T, 128, 256, TRANS_B>(g, task, s, EpilogueStore());
-    if (tm == 256 && tn == 128) return gemm_tile<T, 256, 128, TRANS_B>(g, task, s, EpilogueStore());
-    return gemm_tile<T, 128, 128, TRANS_B>(g, task, s, EpilogueStore());
+    if (tm == 256 && tn == 256) return gemm_body<T, 256, 256, TRANS_B>(op_index, task, tid);
+    if (tm == 128 && tn == 256) return gemm_body<T, 128, 256, TRANS_B>(op_index, task, tid);
+    if (tm == 256 && tn == 128) return gemm_body<T, 256, 128, TRANS_B>(op_index, task, tid);
+    return gemm_body<T, 128, 128, TRANS_B>(op_index, task, tid);
 }
 
-// FAM is the set of op families compiled into this kernel variant.  The families
-// differ widely in register need (a 256x256 GEMM tile takes nearly the whole
-// budget of a two-waves-per-SIMD workgroup); compiled together they share one
-// register allocation, and the row and elementwise bodies then spill values
-// that live across the task loop and reload them in their inner loops.  A
-// plan runs on the smallest variant that holds its families.
-// Returns the task index for the ops that follow in the same fused task: `task` itself, except
-// behind a matmul that splits K, where it is the tile this workgroup finished or -1 (none).
-template <int FAM>
-__device__ __forceinline__ int run_op(const DevOp *op, int task, const Slot &s_in) {
-    // For the long-running bodies the thread index is made opaque per task: the per-lane
-    // addresses they derive from it would otherwise be hoisted out of the task and step
-    // loops as invariants and stay in registers across every other body.  The short
-    // bodies keep theirs hoisted (they run many tasks per step).
-    Slot s = s_in;
-    const int kind = load_const(&op->kind);
-    if (kind == DEV_GEMM || kind == DEV_ATTN || kind == DEV_GEMV) asm volatile("" : "+v"(s.tid));
-    switch (kind) {
-        case DEV_ROW:
-            if (load_const(&op->row.red_len) > 0) {
-                if constexpr ((FAM & FAM_EXT) != 0) {
-                    const RowOpDesc d = load_const(&op->row);
-                    reduce_axis_dispatch(d, task, s);
-                }
-            } else if constexpr ((FAM & FAM_ROW) != 0) {
-                const RowOpDesc d = load_const(&op->row);
-                row_op_dispatch(d, task, s);
-            }
-            break;
-        case DEV_EWISE:
-            if constexpr ((FAM & FAM_EWISE) != 0) {
-                const EwiseDesc d = load_const(&op->ew);
-                ewise_dispatch(d, task, s);
-            }
-            break;
-        case DEV_GEMM:
-            if (load_const(&op->gemm.dtype) == 0 || load_const(&op->gemm.trans_a) != 0) {
-                if constexpr ((FAM & FAM_EXT) != 0) {
-                    const GemmDesc g = load_const(&op->gemm);
-                    if (g.dtype == 0) gemm_f32_dispatch(g, task, s);
-                    else if (g.dtype == 1) {
-                        if (g.trans_b) gemm_tile<f16, 128, 128, true, EpilogueStore, true>(g, task, s, EpilogueStore());
-                        else gemm_tile<f16, 128, 128, false, EpilogueStore, true>(g, task, s, EpilogueStore());
-                    } else {
-                        if (g.trans_b) gemm_tile<bf16, 128, 128, true, EpilogueStore, true>(g, task, s, EpilogueStore());
-                        else gemm_tile<bf16, 128, 128, false, EpilogueStore, true>(g, task, s, EpilogueStore());
-                    }
-                }
-            } else if constexpr ((FAM & FAM_GEMM) != 0) {
-                const bool trans_b = load_const(&op->gemm.trans_b) != 0;
-                if (load_const(&op->gemm.dtype) == 1) {
-                    if (trans_b) return gemm_by_tile<FAM, f16, true>(op, task, s);
-                    return gemm_by_tile<FAM, f16, false>(op, task, s);
-                } else {
-                    if (trans_b) return gemm_by_tile<FAM, bf16, true>(op, task, s);
-                    return gemm_by_tile<FAM, bf16, false>(op, task, s);
-                }
-            }
-            break;
-        case DEV_GEMV:
-            if constexpr ((FAM & FAM_GEMV) != 0) {
-                const GemvDesc d = load_const(&op->gemv);
-                gemv_dispatch(d, task, s);
-            }
-            break;
-        case DEV_EMBED:
+// The first op of a task, of the long-running kind KIND, for one task.  Returns (uniformly) the
+// task index for the ops that follow in the same fused task: `task` itself, except behind a
+// matmul that splits K, where it is the tile this workgroup finished or -1 (none).
+template <int FAM, int KIND>
+__device__ __forceinline__ int run_long(int op_index, int task, int tid) {
+    const DevOp *op = KARG(prog.ops) + op_index;
+    int follow = task;
+    if constexpr (KIND == DEV_GEMM) {
+        const int dtype = load_const(&op->gemm.dtype);
+        const bool trans_a = load_const(&op->gemm.trans_a) != 0, trans_b = load_const(&op->gemm.trans_b) != 0;
+        if (dtype == 0 || trans_a) {
             if constexpr ((FAM & FAM_EXT) != 0) {
-                const EmbedDesc d = load_const(&op->emb);
-                embedding_task(d, task, s);
+                if (dtype == 0) gemm_f32_body(op_index, task, tid);
+                else if (dtype == 1) {
+                    if (trans_b) gemm_body<f16, 128, 128, true, true>(op_index, task, tid);
+                    else gemm_body<f16, 128, 128, false, true>(op_index, task, tid);
+                } else {
+                    if (trans_b) gemm_body<bf16, 128, 128, true, true>(op_index, task, tid);
+                    else gemm_body<bf16, 128, 128, false, true>(op_index, task, tid);
+                }
             }
-            break;
-        case DEV_ATTN:
-            if constexpr ((FAM & FAM_ATTN) != 0) {
-                const AttnDesc d = load_const(&op->attn);
-                attn_dispatch(d, task, s);
+        } else if constexpr ((FAM & FAM_GEMM) != 0) {
+            if (dtype == 1) {
+                follow = trans_b ? gemm_by_tile<FAM, f16, true>(op, op_index, task, tid)
+                                 : gemm_by_tile<FAM, f16, false>(op, op_index, task, tid);
+            } else {
+                follow = trans_b ? gemm_by_tile<FAM, bf16, true>(op, op_index, task, tid)
+                                 : gemm_by_tile<FAM, bf16, false>(op, op_index, task, tid);
             }
-            break;
-        default: break;
+            follow = __builtin_amdgcn_readfirstlane(follow);
+        }
+    } else if constexpr (KIND == DEV_GEMV) {
+        if constexpr ((FAM & FAM_GEMV) != 0) gemv_body(op_index, task, tid);
+    } else if constexpr (KIND == DEV_ATTN) {
+        if constexpr ((FAM & FAM_ATTN) != 0) attn_body(op_index, task, tid);
     }
-    return task;
+    return follow;
 }
 
-// task_seq<> of the reference, parameters read from the table
-// (kernel_template.in:11-27).
+// The tasks of one task_seq<> of the reference (kernel_template.in:11-27: task ids dealt to
+// processors and slots by the formula): the group's parameters and this workgroup's share.
+struct TaskDeal {
+    DevTaskGroup g;
+    int64_t base;   // id of this workgroup's first task
+    int64_t round;  // id step per full deal
+    bool mine;      // this workgroup is in the group's processor range
+};
+
+__device__ __forceinline__ TaskDeal deal_of(int gi) {
+    TaskDeal d;
+    d.g = load_const(KARG(prog.groups) + gi);
+    const DevTaskGroup &g = d.g;
+    const int block = blockIdx.x, grid = gridDim.x;
+    d.mine = in_range(block, g.proc_b, g.proc_e, g.proc_s);
+    const int n_procs = (g.proc_e - g.proc_b + g.proc_s - 1) / g.proc_s;
+    const int p = ((block + grid - g.proc_cur) % grid) / g.proc_s;
+    // Task ids fit 32 bits (the host rejects larger plans); 64-bit products only
+    // where the formula could overflow before the range check.
+    d.base = g.task_b + (int64_t)p * g.task_s * g.gran;
+    d.round = (int64_t)g.task_s * g.gran * n_procs;
+    return d;
+}
+
+__device__ __forceinline__ int64_t task_id(const TaskDeal &d, unsigned t) {
+    if (d.g.gran == 1) return d.base + d.round * t;
+    const unsigned q = t / (unsigned)d.g.gran, r = t - q * (unsigned)d.g.gran;
+    return d.base + (int64_t)d.g.task_s * r + d.round * q;
+}
+
+// Before task index `ti` of a consumer group: wait until the producers' row blocks it reads
+// are complete in this iteration.  The data is then read through this XCD's L2 without
+// invalidating it: the host admits the wait in place of a barrier only where no workgroup can
+// have fetched these lines since the last barrier (rows own whole cache lines, and every reader
+// in between waits like this one).  False (uniformly) once `abort` is raised.
+__device__ __forceinline__ bool wait_for_rows(const DevTaskGroup &g, int ti, const Slot &s, unsigned epoch) {
+    volatile int *fail = reinterpret_cast<volatile int *>(g_loop_lds) + 1;
+    const DevWait *waits = KARG(prog.waits) + g.wait_begin;
+    const int32_t *spans = KARG(prog.wait_spans) + g.span_begin + 2 * (ti * g.n_waits);
+    unsigned *counters = KARG(prog.dep_counters);
+    LoopControl *ctl = KARG(ctl);
+    const uint64_t limit = KARG(wait_ticks);
+    bool ok = true;
+    for (int w = 0; w < g.n_waits; ++w) {
+        const DevWait dw = load_const(waits + w);
+        const int lo = load_const(spans + 2 * w), hi = load_const(spans + 2 * w + 1);
+        const unsigned target = (unsigned)dw.expect * epoch;
+        for (int c = lo + s.tid; c <= hi; c += s.nthreads)
+            ok = poll_reached(counters + (size_t)(dw.counter_base + c) * kDepStride, target, ctl, limit) && ok;
+    }
+    if (!ok) *fail = 1;
+    __syncthreads();
+    return *fail == 0;
+}
+
+// After task index `ti` of a producer group: every wave's stores have been acknowledged by the
+// L2, the L2 is written back (the release), then the row block's counter grows by one.
+__device__ __forceinline__ void signal_rows(const DevTaskGroup &g, int ti) {
+    drain_stores_then_barrier();
+    if (threadIdx.x == 0) {
+        const int block = load_const(KARG(prog.signal_map) + g.signal_begin + ti);
+        __hip_atomic_fetch_add(KARG(prog.dep_counters) + (size_t)(g.signal_base + block) * kDepStride, 1u,
+                               __ATOMIC_RELEASE, AGENT);
+    }
+}
+
+__device__ __forceinline__ int task_index(const DevTaskGroup &g, int64_t id) {
+    return ((int)id - g.task_b) / g.task_s;
+}
+
+__device__ __forceinline__ void trace_task(const DevTaskGroup &g, int64_t id, int slot_k, int order, const Slot &s) {
+#ifndef ARKMI_NO_TRACE
+    TraceRecord *trace = KARG(prog.trace);
+    if (trace && g.trace_offset >= 0 && s.tid == 0) {
+        TraceRecord rec{(int)blockIdx.x, slot_k, order};
+        trace[g.trace_offset + task_index(g, id)] = rec;
+    }
+#endif
+}
+
+// The task loop of a group of small ops: the group's parameters stay in registers.
 template <int FAM>
-__device__ __forceinline__ void run_group(const LoopProgram &prog, const DevTaskGroup *gptr) {
-    const DevTaskGroup g = load_const(gptr);
-    const int block = blockIdx.x;
-    if (!in_range(block, g.proc_b, g.proc_e, g.proc_s)) return;
-    const DevOp *ops = prog.ops + g.op_begin;
+__device__ __forceinline__ bool run_small_tasks(int gi, const TaskDeal &d, const Slot &s, int slot_k, unsigned epoch) {
+    const DevTaskGroup &g = d.g;
+    const DevOp *ops = KARG(prog.ops) + g.op_begin;
+    const bool deps = KARG(prog.dep_counters) != nullptr;
+    const bool waits = deps && g.n_waits > 0, signals = deps && g.signal_begin >= 0;
+    int order = 0;
+    for (unsigned t = (unsigned)slot_k;; t += (unsigned)g.n_slots, ++order) {
+        const int64_t id = task_id(d, t);
+        if (id >= g.task_e) break;
+        const int ti = (waits || signals) ? task_index(g, id) : 0;
+        trace_task(g, id, slot_k, order, s);
+        if (waits && !wait_for_rows(g, ti, s, epoch)) return false;
+        for (int o = 0; o < g.op_count; ++o) {
+            // later ops of a fused task read what earlier ones of the same workgroup wrote:
+            // the workgroup meets (its waves share one L1, which sees their stores)
+            if (o > 0) s.sync();
+            run_small<FAM>(ops + o, (int)id, s);
+        }
+        if (signals) signal_rows(g, ti);
+    }
+    return true;
+}
+
+// The task loop of a group whose first op is long-running (KIND: matmul, skinny matmul,
+// attention), one loop per kind, so what the compiler lifts out of a loop stays live across
+// that body only.  Nothing of the group's parameters is kept across the body: they are read
+// again for every task.
+template <int FAM, int KIND>
+__device__ __forceinline__ bool run_long_tasks(int gi, const Slot &s, int slot_k, unsigned epoch) {
+    int order = 0;
+    for (unsigned t = (unsigned)slot_k;; ++order) {
+        int follow;
+        {
+            const TaskDeal d = deal_of(gi);
+            const DevTaskGroup &g = d.g;
+            const int64_t id = task_id(d, t);
+            if (id >= g.task_e) break;
+            const bool deps = KARG(prog.dep_counters) != nullptr;
+            trace_task(g, id, slot_k, order, s);
+            if (deps && g.n_waits > 0 && !wait_for_rows(g, task_index(g, id), s, epoch)) return false;
+            follow = run_long<FAM, KIND>(g.op_begin, (int)id, s.tid);  // uniform across the workgroup
+        }
+        const DevTaskGroup g = load_const(KARG(prog.groups) + gi);
+        if constexpr (KIND == DEV_GEMM) {
+            const DevOp *ops = KARG(prog.ops) + g.op_begin;
+            for (int o = 1; o < g.op_count && follow >= 0; ++o) {
+                s.sync();
+                run_follower<FAM>(ops + o, follow, s);
+            }
+        }
+        // (a matmul that splits K signals for the tile this workgroup finished, if any)
+        if (KARG(prog.dep_counters) != nullptr && g.signal_begin >= 0 && follow >= 0)
+            signal_rows(g, task_index(g, follow));
+        t += (unsigned)g.n_slots;
+    }
+    return true;
+}
+
+template <int FAM>
+__device__ __forceinline__ bool run_group(int gi, unsigned epoch) {
+    const TaskDeal d = deal_of(gi);
+    const DevTaskGroup &g = d.g;
+    if (!d.mine) return true;
     const int slot_threads = g.slot_warps * kWave;
     const int k = threadIdx.x / slot_threads;
-    if (k >= g.n_slots) return;
-    const int n_procs = (g.proc_e - g.proc_b + g.proc_s - 1) / g.proc_s;
-    const int grid = gridDim.x;
-    const int p = ((block + grid - g.proc_cur) % grid) / g.proc_s;
+    if (k >= g.n_slots) return true;
     Slot s;
     s.tid = threadIdx.x - k * slot_threads;
     s.nthreads = slot_threads;
     s.lds = (lds_ptr)g_loop_lds + kLdsReserved + k * g.slot_sram;
     s.lds_bytes = g.slot_sram;
     s.whole_block = (slot_threads == (int)blockDim.x);
-    // Task ids fit 32 bits (the host rejects larger plans); 64-bit products only
-    // where the formula could overflow before the range check.
-    const int64_t base = g.task_b + (int64_t)p * g.task_s * g.gran;
-    const int64_t round = (int64_t)g.task_s * g.gran * n_procs;  // id step per full deal
-    int order = 0;
-    for (unsigned t = (unsigned)k;; t += (unsigned)g.n_slots, ++order) {
-        int64_t id;
-        if (g.gran == 1) {
-            id = base + round * t;
-        } else {
-            const unsigned q = t / (unsigned)g.gran, r = t - q * (unsigned)g.gran;
-            id = base + (int64_t)g.task_s * r + round * q;
-        }
-        if (id >= g.task_e) break;
-#ifndef ARKMI_NO_TRACE
-        if (prog.trace && g.trace_offset >= 0 && s.tid == 0) {
-            TraceRecord rec{block, k, order};
-            prog.trace[g.trace_offset + (int)((id - g.task_b) / g.task_s)] = rec;
-        }
-#endif
-        int follow = (int)id;  // uniform across the workgroup
-        for (int o = 0; o < g.op_count && follow >= 0; ++o) {
-            if (o > 0) {
-                // later ops of a fused task read what earlier ones wrote: the stores
-                // have reached the L2, and the L1 must not serve older copies
-                s.sync();
-                if (s.tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-                s.sync();
-            }
-            follow = run_op<FAM>(ops + o, follow, s);
-        }
+    // one task loop per long-running kind of first op, one for the tasks of small ops
+    // (a variant holds the loops of the families it was built for)
+    const int first = load_const(&(KARG(prog.ops) + g.op_begin)->kind);
+    if constexpr ((FAM & (FAM_GEMM | FAM_SPLITK | FAM_EXT)) != 0) {
+        if (first == DEV_GEMM) return run_long_tasks<FAM, DEV_GEMM>(gi, s, k, epoch);
     }
+    if constexpr ((FAM & FAM_GEMV) != 0) {
+        if (first == DEV_GEMV) return run_long_tasks<FAM, DEV_GEMV>(gi, s, k, epoch);
+    }
+    if constexpr ((FAM & FAM_ATTN) != 0) {
+        if (first == DEV_ATTN) return run_long_tasks<FAM, DEV_ATTN>(gi, s, k, epoch);
+    }
+    if constexpr ((FAM & (FAM_ROW | FAM_EWISE | FAM_EXT)) != 0) {
+        if (first != DEV_GEMM && first != DEV_GEMV && first != DEV_ATTN)
+            return run_small_tasks<FAM>(gi, d, s, k, epoch);
+    }
+    return true;
 }
 
+// One iteration of the plan's body; `epoch` counts the iterations since the launch from 1.
 template <int FAM>
-__device__ __forceinline__ bool run_body(const LoopProgram &prog, LoopControl *ctl, XcdInfo &xi,
-                                          uint64_t wait_ticks) {
-    const bool clocked = prog.step_clock && threadIdx.x == 0;
-    unsigned long long *clk = prog.step_clock + (size_t)blockIdx.x * (prog.num_steps + 1);
-    for (int si = 0; si < prog.num_steps; ++si) {
-        const DevStep st = load_const(prog.steps + si);
-        if (clocked) clk[si] = wall_clock64();
+__device__ __forceinline__ bool run_body(XcdInfo &xi, unsigned epoch) {
+    for (int si = 0; si < KARG(prog.num_steps); ++si) {
+        const DevStep st = load_const(KARG(prog.steps) + si);
+        unsigned long long *clock = KARG(prog.step_clock);
+        if (clock && threadIdx.x == 0) clock[(size_t)blockIdx.x * (KARG(prog.num_steps) + 1) + si] = wall_clock64();
         if (st.kind == STEP_BARRIER) {
+            LoopControl *ctl = KARG(ctl);
             if ((unsigned)st.count == gridDim.x) {
-                if (!grid_barrier_xcd(ctl, xi, wait_ticks)) return false;
+                if (!grid_barrier_xcd(ctl, xi, KARG(wait_ticks))) return false;
             } else if (in_range(blockIdx.x, st.b, st.e, st.s)) {
-                if (!grid_barrier(&ctl->bars[st.index], (unsigned)st.count, ctl, wait_ticks))
-                    return false;
+                if (!grid_barrier(&ctl->bars[st.index], (unsigned)st.count, ctl, KARG(wait_ticks))) return false;
             }
         } else if (st.kind == STEP_LOCAL_SYNC) {
-            // this workgroup's stores have reached the L2 it shares with nobody else
-            // for these lines; drop what its L1 still holds of them
-            __syncthreads();
-            if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+            // the next group reads only what this workgroup itself wrote: its waves share one
+            // L1, which sees their own stores, so the workgroup only has to meet
             __syncthreads();
         } else {
-            run_group<FAM>(prog, prog.groups + st.index);
+            if (!run_group<FAM>(st.index, epoch)) return false;
         }
     }
-    if (clocked) clk[prog.num_steps] = wall_clock64();
+    unsigned long long *clock = KARG(prog.step_clock);
+    if (clock && threadIdx.x == 0) {
+        const int n = KARG(prog.num_steps);
+        clock[(size_t)blockIdx.x * (n + 1) + n] = wall_clock64();
+    }
     return true;
 }
 
 template <int FAM>
-__global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(
-    LoopProgram prog, LoopControl *ctl, HostMailbox *mb, int one_shot_iters, uint64_t idle_ticks,
-    uint64_t wait_ticks) {
+__global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(LoopArgs) {
     const unsigned nblocks = gridDim.x;
     const bool leader = (blockIdx.x == 0 && threadIdx.x == 0);
+    // LDS control words: [0] the barriers' verdict, [1] raised when a dependency wait gave up
+    if (threadIdx.x == 0) reinterpret_cast<volatile int *>(g_loop_lds)[1] = 0;
     // count the workgroups per XCD (the control block is zeroed before every launch)
     XcdInfo xi;
     xi.epoch = 0;
     xi.x = xcc_id();
-    if (threadIdx.x == 0) __hip_atomic_fetch_add(&ctl->xcd_blocks[xi.x], 1u, __ATOMIC_RELAXED, AGENT);
-    if (!grid_barrier(&ctl->all, nblocks, ctl, wait_ticks)) {
-        if (threadIdx.x == 0) {
-            __hip_atomic_store(&mb->status, (int)MB_ABORTED, __ATOMIC_RELAXED, SYSTEM);
-            if (blockIdx.x == 0) __hip_atomic_store(&mb->alive, 0, __ATOMIC_RELEASE, SYSTEM);
+    {
+        LoopControl *ctl = KARG(ctl);
+        HostMailbox *mb = KARG(mb);
+        if (threadIdx.x == 0) __hip_atomic_fetch_add(&ctl->xcd_blocks[xi.x], 1u, __ATOMIC_RELAXED, AGENT);
+        if (!grid_barrier(&ctl->all, nblocks, ctl, KARG(wait_ticks))) {
+            if (threadIdx.x == 0) {
+                __hip_atomic_store(&mb->status, (int)MB_ABORTED, __ATOMIC_RELAXED, SYSTEM);
+                if (blockIdx.x == 0) __hip_atomic_store(&mb->alive, 0, __ATOMIC_RELEASE, SYSTEM);
+            }
+            return;
         }
-        return;
+        xi.nx = __hip_atomic_load(&ctl->xcd_blocks[xi.x], __ATOMIC_RELAXED, AGENT);
+        xi.nxcd = 0;
+        for (int i = 0; i < kMaxXcds; ++i)
+            xi.nxcd += __hip_atomic_load(&ctl->xcd_blocks[i], __ATOMIC_RELAXED, AGENT) ? 1u : 0u;
     }
-    xi.nx = __hip_atomic_load(&ctl->xcd_blocks[xi.x], __ATOMIC_RELAXED, AGENT);
-    xi.nxcd = 0;
-    for (int i = 0; i < kMaxXcds; ++i)
-        xi.nxcd += __hip_atomic_load(&ctl->xcd_blocks[i], __ATOMIC_RELAXED, AGENT) ? 1u : 0u;
+    unsigned epoch = 0;  // iterations of the body started since the launch
     for (;;) {
         int iter;
+        const int one_shot_iters = KARG(one_shot_iters);
         if (one_shot_iters > 0) {
             iter = one_shot_iters;
         } else {
+            LoopControl *ctl = KARG(ctl);
             if (leader) {
+                HostMailbox *mb = KARG(mb);
+                const uint64_t idle_ticks = KARG(idle_ticks);
                 const uint64_t t0 = wall_clock64();
                 int cmd;
                 unsigned polls = 0;
@@ -393,10 +599,11 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(
                 }
                 __hip_atomic_store(&ctl->iter, cmd, __ATOMIC_RELAXED, AGENT);
             }
-            if (!grid_barrier_xcd(ctl, xi, wait_ticks)) break;
+            if (!grid_barrier_xcd(ctl, xi, KARG(wait_ticks))) break;
             iter = __hip_atomic_load(&ctl->iter, __ATOMIC_RELAXED, AGENT);
             if (iter < 0) {
                 if (leader) {
+                    HostMailbox *mb = KARG(mb);
                     if (iter == -2) __hip_atomic_store(&mb->status, (int)MB_IDLE_EXIT, __ATOMIC_RELAXED, SYSTEM);
                     __hip_atomic_store(&mb->alive, 0, __ATOMIC_RELEASE, SYSTEM);
                 }
@@ -409,30 +616,32 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(
                 // the host has compared the end of the body with its start: a barrier
                 // when another workgroup's data is involved, a local sync when only
                 // this workgroup's own, nothing when the iterations share no data
-                if (prog.iter_sync == 2) {
-                    ok = grid_barrier_xcd(ctl, xi, wait_ticks);
-                } else if (prog.iter_sync == 1) {
-                    __syncthreads();
-                    if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+                const int iter_sync = KARG(prog.iter_sync);
+                if (iter_sync == 2) {
+                    ok = grid_barrier_xcd(KARG(ctl), xi, KARG(wait_ticks));
+                } else if (iter_sync == 1) {
                     __syncthreads();
                 }
             }
-            if (ok) ok = run_body<FAM>(prog, ctl, xi, wait_ticks);
+            ++epoch;
+            if (ok) ok = run_body<FAM>(xi, epoch);
         }
         if (!ok) break;
         // results must be visible to the host before the command is cleared: every
         // wave's stores are in the L2 before thread 0's system-scope release
         drain_stores_then_barrier();
         if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "");
-        if (!grid_barrier_xcd(ctl, xi, wait_ticks)) break;
+        if (!grid_barrier_xcd(KARG(ctl), xi, KARG(wait_ticks))) break;
         if (one_shot_iters > 0) return;
         if (leader) {
+            HostMailbox *mb = KARG(mb);
             __hip_atomic_store(&mb->done, mb->done + iter, __ATOMIC_RELAXED, SYSTEM);
             __hip_atomic_store(&mb->cmd, 0, __ATOMIC_RELEASE, SYSTEM);
         }
     }
     // a bounded wait expired somewhere: report and leave
     if (threadIdx.x == 0) {
+        HostMailbox *mb = KARG(mb);
         __hip_atomic_store(&mb->status, (int)MB_ABORTED, __ATOMIC_RELAXED, SYSTEM);
         if (blockIdx.x == 0) __hip_atomic_store(&mb->alive, 0, __ATOMIC_RELEASE, SYSTEM);
     }
@@ -440,10 +649,12 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(
 
 // One task group as a kernel of its own (no loop, no barriers): the same op
 // bodies launched the conventional way, one kernel per op, for comparison with
-// the persistent loop kernel.
+// the persistent loop kernel.  The host passes no dependency counters here: kernel
+// boundaries order everything.
 template <int FAM>
-__global__ __launch_bounds__(kLoopMaxThreads) void arkmi_step_kernel(LoopProgram prog, int group) {
-    run_group<FAM>(prog, prog.groups + group);
+__global__ __launch_bounds__(kLoopMaxThreads) void arkmi_step_kernel(LoopArgs) {
+    if (threadIdx.x == 0) reinterpret_cast<volatile int *>(g_loop_lds)[1] = 0;
+    run_group<FAM>(KARG(group), 1u);
 }
 
 // Defines the host-visible handles of one kernel variant; each variant is its own

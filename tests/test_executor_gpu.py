@@ -913,3 +913,50 @@ def test_matmul_split_k_with_follower_and_neighbours(oracle):
     ref = oracle.unary(oracle.binary(np.ascontiguousarray(r[pick]), oracle.matmul(xs_ref, w, dtype, trans_b=True),
                                      "add", dtype), "relu", dtype)
     close(oracle, ref, got[pick], dtype, 1e-2)
+
+
+# ---------------------------------------------------------------- caches across iterations
+def test_follower_sees_this_iterations_tile_not_a_cached_one(oracle):
+    """x <- 0.5 * relu(x @ w), the relu fused behind the matmul: every iteration the follower reads a
+    tile its own workgroup has just rewritten with new values, small enough to sit in the CU's L1 from
+    the iteration before.  A stale read would feed the previous iteration's tile forward."""
+    from ark_amd import Model
+    dtype, n = "fp16", 128
+    x = make(oracle, (n, n), dtype, 121, "uniform")
+    w = make(oracle, (n, n), dtype, 122, "normal", scale=2.0 / np.sqrt(n))
+    m = Model()
+    tx, tw = m.tensor([n, n], dtype), m.tensor([n, n], dtype)
+    with m.planner_context(sync=False):
+        z = m.relu(m.matmul(tx, tw))
+    m.mul(z, 0.5, tx)
+    iters = 6
+    (got,), ex, plan = run_model(m, {tx: x, tw: w}, [tx], iters=iters)
+    assert len(json.loads(plan)["TaskInfos"][0]["Ops"]) == 2
+    want = x
+    for _ in range(iters):
+        want = oracle.scalar(oracle.unary(oracle.matmul(want, w, dtype), "relu", dtype), 0.5, "mul", dtype)
+    t, g = (oracle.to_f32(a, dtype).astype(np.float64) for a in (want, got))
+    assert np.abs(t).max() > 1e-3  # the sequence has not died out
+    assert np.abs(t - g).max() <= 1e-2 * np.abs(t).max()
+
+
+def test_grid_barrier_drops_other_workgroups_old_lines_from_the_l1(oracle):
+    """a <- transpose(a) + 1 on a 16 KB tensor cut into 8 tasks: every workgroup re-reads, each
+    iteration, a few lines that other workgroups have rewritten since, and that still sit in its own L1
+    from the iteration before.  The grid barrier between the two ops must drop them."""
+    from ark_amd import Model
+    a = make(oracle, (1, 1, 64, 64), "fp32", 123)
+    cfg = {"NumWarps": 8, "SramBytes": 0, "Tile": [8, 64], "NumTasks": 8}
+    m = Model()
+    ta = m.tensor(a.shape, "fp32")
+    with m.planner_context(config=cfg):
+        tb = m.transpose(ta, [0, 1, 3, 2])
+    with m.planner_context(config=cfg):
+        m.add(tb, 1.0, ta)
+    iters = 7
+    (got,), ex, _ = run_model(m, {ta: a}, [ta], iters=iters)
+    assert ex.info()["iteration_sync"] == 2 and ex.info()["barriers_local"] == 0
+    want = a.copy()
+    for _ in range(iters):
+        want = np.ascontiguousarray(want.transpose(0, 1, 3, 2)) + np.float32(1.0)
+    assert np.array_equal(got, want)
