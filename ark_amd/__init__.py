@@ -8,3 +8,8 @@ from ._lib import lib, check, ArkmiError, DTYPES, device_info  # noqa: F401
 from . import ops  # noqa: F401
 from .model import Model, Tensor, PlannerContext, reset_ids  # noqa: F401
 from .executor import Executor, plan_schedule, schedule_tasks  # noqa: F401
+
+
+def init():
+    """ark::init(): read the ARK_* environment variables again."""
+    check(lib().arkmi_init())

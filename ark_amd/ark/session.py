@@ -256,7 +256,9 @@ class Module:
 
 
 def init():
-    """Drops the global model and destroys a live executor."""
+    """Drops the global model, destroys a live executor and reads the ARK_* environment again."""
+    from .._lib import lib, check
+    check(lib().arkmi_init())
     Model.reset()
     ex = _RuntimeState.executor
     if ex is not None:

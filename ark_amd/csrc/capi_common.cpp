@@ -4,6 +4,7 @@
 #include <mutex>
 
 #include "host_common.h"
+#include "host/ir.hpp"
 
 namespace arkmi {
 
@@ -38,6 +39,10 @@ extern "C" {
 const char *arkmi_last_error(void) { return arkmi::g_last_error.c_str(); }
 
 const char *arkmi_version(void) { return "0.1.0"; }
+
+int arkmi_init(void) {
+    return arkmi::guard([&] { ark::reload_env(); });
+}
 
 int arkmi_device_info_get(int device_id, arkmi_device_info *out) {
     return arkmi::guard([&] {

@@ -812,6 +812,250 @@ bool same_decomposition(const Json &ti_a, const ScheduleStep &sa, const Json &ti
 }  // namespace
 
 // ---------------------------------------------------------------------------
+// per-task dependency counters (host side)
+// ---------------------------------------------------------------------------
+// A grid barrier orders every workgroup after every other.  Where everything that crosses it
+// is a read of rows that tasks of an earlier group wrote, and both ops are of a kind whose
+// tasks map to row ranges of one 2-D row space, the barrier is replaced by counters in device
+// memory: a producer task adds one to the counter of the row block it completed (after a
+// write-back of its L2), a consumer task waits until the counters of the blocks it reads have
+// reached what one iteration contributes times the iteration number.
+namespace {
+
+using RowSpan = std::function<void(int, int64_t &, int64_t &)>;  // task index -> rows [r0, r1)
+
+// One operand of an op as rows of a 2-D row space.
+struct RowAccess {
+    const char *ptr = nullptr;  // address of row 0
+    int64_t pitch = 0;          // bytes between rows
+    int64_t width = 0;          // bytes of a row the op touches (<= pitch)
+    int64_t rows = 0;
+    bool write = false;
+    RowSpan span;
+};
+
+// Row accesses of one lowered op; an operand whose tasks do not map to row ranges is left out.
+std::vector<RowAccess> row_accesses(const DevOp &op, int slot_warps) {
+    std::vector<RowAccess> v;
+    auto add = [&](const void *p, int64_t pitch, int64_t width, int64_t rows, bool write, RowSpan span) {
+        if (!p || pitch <= 0 || rows <= 0 || width <= 0 || (width > pitch && rows > 1)) return;
+        RowAccess a;
+        a.ptr = static_cast<const char *>(p); a.pitch = pitch; a.width = std::min(width, pitch); a.rows = rows;
+        a.write = write; a.span = std::move(span);
+        v.push_back(std::move(a));
+    };
+    if (op.kind == DEV_ROW && op.row.red_len == 0) {
+        const RowOpDesc &r = op.row;
+        const int64_t elem = r.dtype == 0 ? 4 : 2;
+        // rows r = (n, c, h) are equally spaced when the outer strides nest
+        auto nested = [&](const int64_t s[3]) {
+            const int64_t n = r.rows / std::max<int64_t>(1, (int64_t)r.dim_c * r.dim_h);
+            if (r.dim_h > 1 && s[2] <= 0) return false;
+            if (r.dim_c > 1 && s[1] != (int64_t)r.dim_h * s[2]) return false;
+            if (n > 1 && s[0] != (int64_t)r.dim_c * r.dim_h * s[2]) return false;
+            return s[2] > 0;
+        };
+        const int64_t per_task = (int64_t)slot_warps * std::max(1, r.rows_per_wave);
+        const int64_t rows = r.rows;
+        RowSpan span = [per_task, rows](int t, int64_t &r0, int64_t &r1) {
+            r0 = std::min<int64_t>(rows, (int64_t)t * per_task);
+            r1 = std::min<int64_t>(rows, r0 + per_task);
+        };
+        const bool reduce = r.kind == ROW_SUM || r.kind == ROW_MAX || r.kind == ROW_MEAN;
+        if (nested(r.in_s)) add(r.in, r.in_s[2] * elem, (int64_t)r.cols * elem, rows, false, span);
+        if (nested(r.out_s)) add(r.out, r.out_s[2] * elem, (reduce ? 1 : (int64_t)r.cols) * elem, rows, true, span);
+    } else if (op.kind == DEV_GEMM && op.gemm.dtype != 0 && !op.gemm.trans_a && op.gemm.batch_total == 1) {
+        const GemmDesc &g = op.gemm;
+        const int bm = op.gemm_tile_m, tiles_n = g.tiles_n, tiles = g.tiles_m * g.tiles_n;
+        auto rows_of = [bm, tiles_n, tiles](int64_t limit) -> RowSpan {
+            return [bm, tiles_n, tiles, limit](int t, int64_t &r0, int64_t &r1) {
+                const int tm = (t % tiles) / tiles_n;
+                r0 = std::min<int64_t>(limit, (int64_t)tm * bm);
+                r1 = std::min<int64_t>(limit, r0 + bm);
+            };
+        };
+        const int64_t n_out = g.b2 ? g.n / 2 : g.n;
+        add(g.a, (int64_t)g.lda * 2, (int64_t)g.k * 2, g.m, false, rows_of(g.m));
+        add(g.c, (int64_t)g.ldc * 2, n_out * 2, g.store_m, true, rows_of(g.store_m));
+        const int64_t k = g.k;
+        if (!g.trans_b) {  // [K, N]: every task reads every row
+            add(g.b, (int64_t)g.ldb * 2, (int64_t)g.n * 2, k, false, [k](int, int64_t &r0, int64_t &r1) { r0 = 0; r1 = k; });
+        } else {           // [N, K]: the task's columns are rows of the operand
+            const int bn = g.b2 ? op.gemm_tile_n / 2 : op.gemm_tile_n;
+            RowSpan cols = [bn, tiles_n, tiles, n_out](int t, int64_t &r0, int64_t &r1) {
+                const int tn = (t % tiles) % tiles_n;
+                r0 = std::min<int64_t>(n_out, (int64_t)tn * bn);
+                r1 = std::min<int64_t>(n_out, r0 + bn);
+            };
+            add(g.b, (int64_t)g.ldb * 2, k * 2, n_out, false, cols);
+            if (g.b2) add(g.b2, (int64_t)g.ldb * 2, k * 2, n_out, false, cols);
+        }
+    } else if (op.kind == DEV_EWISE && op.ew.shape[0] * op.ew.shape[1] == 1) {
+        const EwiseDesc &e = op.ew;
+        const int64_t rows = e.shape[2], cols = e.shape[3];
+        const int th = e.tile_h, tiles_h = e.tiles_h, tiles_w = e.tiles_w;
+        RowSpan span = [rows, th, tiles_h, tiles_w](int t, int64_t &r0, int64_t &r1) {
+            const int i = (t / tiles_w) % tiles_h;
+            r0 = std::min<int64_t>(rows, (int64_t)i * th);
+            r1 = std::min<int64_t>(rows, r0 + th);
+        };
+        RowSpan whole = [](int, int64_t &r0, int64_t &r1) { r0 = 0; r1 = 1; };
+        const int64_t es_in = (e.dt_in == 1 || e.dt_in == 2) ? 2 : 4, es_out = (e.dt_out == 1 || e.dt_out == 2) ? 2 : 4;
+        auto operand = [&](const EwTensor &t, int64_t es, bool write, int64_t period) {
+            if (!t.ptr || (t.s[3] != 0 && t.s[3] != 1)) return;
+            const int64_t w = (t.s[3] == 0 ? 1 : period > 0 ? period : cols) * es;
+            if (t.s[2] == 0) add(t.ptr, w, w, 1, write, whole);  // one row every task reads
+            else if (t.s[2] > 0) add(t.ptr, t.s[2] * es, w, rows, write, span);
+        };
+        operand(e.out, es_out, true, 0);
+        if (e.op != EW_SCALAR_ASSIGN) operand(e.in0, es_in, false, 0);
+        operand(e.in1, es_in, false, e.in1_period);
+    } else if (op.kind == DEV_ATTN) {
+        const AttnDesc &a = op.attn;
+        const int QB = a.q_blocks, heads = a.heads, batch = a.batch, causal = a.causal;
+        const int64_t sq = a.seq_q, sk = a.seq_k;
+        auto decode = [QB, heads, batch, causal](int t, int &b, int &qb) {
+            const int bh = t / QB;
+            qb = t - bh * QB;
+            if (causal && bh >= (batch * heads + 1) / 2) qb = QB - 1 - qb;
+            b = bh / heads;
+        };
+        RowSpan q_span = [decode, sq](int t, int64_t &r0, int64_t &r1) {
+            int b, qb;
+            decode(t, b, qb);
+            r0 = (int64_t)b * sq + std::min<int64_t>(sq, (int64_t)qb * kAttnQBlock);
+            r1 = (int64_t)b * sq + std::min<int64_t>(sq, (int64_t)(qb + 1) * kAttnQBlock);
+        };
+        // keys are fetched in whole blocks of kAttnKBlock up to the task's last visible one
+        RowSpan kv_span = [decode, sq, sk, causal](int t, int64_t &r0, int64_t &r1) {
+            int b, qb;
+            decode(t, b, qb);
+            int64_t end = sk;
+            if (causal) {
+                end = std::min<int64_t>(sk, std::min<int64_t>((int64_t)(qb + 1) * kAttnQBlock, sq) + (sk - sq));
+                end = std::min<int64_t>(sk, (std::max<int64_t>(0, end) + kAttnKBlock - 1) / kAttnKBlock * kAttnKBlock);
+            }
+            r0 = (int64_t)b * sk;
+            r1 = r0 + end;
+        };
+        auto rows_ok = [&](const int64_t s[3], int64_t seq) { return s[1] > 0 && (batch == 1 || s[0] == seq * s[1]); };
+        const int64_t w = (int64_t)heads * kAttnD * 2;  // all heads of a position, when they are adjacent
+        auto width = [&](const int64_t s[3]) { return s[2] == kAttnD ? w : (int64_t)0; };
+        if (rows_ok(a.q_s, sq)) add(a.q, a.q_s[1] * 2, width(a.q_s), (int64_t)batch * sq, false, q_span);
+        if (rows_ok(a.k_s, sk)) add(a.k, a.k_s[1] * 2, width(a.k_s), (int64_t)batch * sk, false, kv_span);
+        if (rows_ok(a.v_s, sk)) add(a.v, a.v_s[1] * 2, width(a.v_s), (int64_t)batch * sk, false, kv_span);
+        if (rows_ok(a.o_s, sq)) add(a.o, a.o_s[1] * 2, width(a.o_s), (int64_t)batch * sq, true, q_span);
+    }
+    return v;
+}
+
+// A task group as the dependency analysis sees it.
+struct DepGroup {
+    int sched_step = -1;   // index into the schedule
+    int segment = 0;       // schedule barriers ahead of it
+    int group = -1;        // index into the device task groups
+    int n_tasks = 0;       // tasks of the group
+    int n_signal = 0;      // tasks that finish something (the tiles of a matmul that splits K)
+    bool whole_block = false;
+    std::vector<Access> acc;      // every operand (byte ranges inside buffers)
+    std::vector<RowAccess> rows;  // the operands with a row structure (device addresses)
+    // as a producer: the row block each task completes, set on first use
+    std::vector<int> signal_map;
+    int n_blocks = 0, per_block = 0;
+    int counter_base = -1;
+    // as a consumer: blocks [lo, hi] of each producer it waits for, per task
+    struct Wait {
+        int producer;  // index into the DepGroup list
+        std::vector<std::pair<int, int>> span;
+    };
+    std::vector<Wait> waits;
+};
+
+const RowAccess *row_of(const DepGroup &g, const char *ptr, bool write) {
+    for (const auto &r : g.rows)
+        if (r.ptr == ptr && r.write == write) return &r;
+    return nullptr;
+}
+
+// The row blocks of producer `x` as its write `w` cuts them: every task writes exactly one block
+// of `br` rows, the blocks tile the rows, and every block gets the same number of tasks.
+bool establish_blocks(DepGroup &x, const RowAccess &w, int64_t *br_out) {
+    if (x.n_signal <= 0) return false;
+    int64_t r0, r1, br = 0;
+    w.span(0, r0, r1);
+    br = r1 - r0;
+    if (br <= 0) return false;
+    std::vector<int> map((size_t)x.n_signal);
+    for (int t = 0; t < x.n_signal; ++t) {
+        w.span(t, r0, r1);
+        if (r1 <= r0 || r0 % br != 0 || r1 != std::min(w.rows, r0 + br)) return false;
+        map[(size_t)t] = (int)(r0 / br);
+    }
+    const int n_blocks = (int)((w.rows + br - 1) / br);
+    std::vector<int> count((size_t)n_blocks, 0);
+    for (int b : map) {
+        if (b >= n_blocks) return false;
+        ++count[(size_t)b];
+    }
+    for (int c : count)
+        if (c != count[0] || c == 0) return false;
+    if (x.signal_map.empty()) {
+        x.signal_map = map;
+        x.n_blocks = n_blocks;
+        x.per_block = count[0];
+    } else if (x.signal_map != map || x.n_blocks != n_blocks) {
+        return false;
+    }
+    *br_out = br;
+    return true;
+}
+
+constexpr int64_t kLine = 128;  // bytes of an L2 cache line
+
+// Can the read `ay` of group y wait on counters for the write `ax` of group x?  On success the
+// blocks each task of y waits for are merged into y.waits.
+bool cover_with_counters(std::vector<DepGroup> &groups, int xi, const Access &ax, int yi, const Access &ay,
+                         const char *arena, const std::map<size_t, size_t> &buffer_offset) {
+    DepGroup &x = groups[(size_t)xi], &y = groups[(size_t)yi];
+    if (!ax.write || ay.write || !x.whole_block || !y.whole_block) return false;
+    const RowAccess *w = row_of(x, arena + buffer_offset.at(ax.buffer) + ax.begin, true);
+    const RowAccess *r = row_of(y, arena + buffer_offset.at(ay.buffer) + ay.begin, false);
+    if (!w || !r) return false;
+    // A consumer reads through its L2 without invalidating it: lines it fetched for finished
+    // rows must hold nothing another task still has to write, so rows own whole lines.
+    if ((uintptr_t)w->ptr % kLine || w->pitch % kLine || w->width % kLine) return false;
+    if (w->pitch != r->pitch) return false;
+    const int64_t delta = r->ptr - w->ptr;
+    int64_t shift = delta / w->pitch;
+    if (delta < 0 && shift * w->pitch != delta) --shift;
+    const int64_t col = delta - shift * w->pitch;
+    if (col + r->width > w->pitch) return false;
+    int64_t br = 0;
+    if (!establish_blocks(x, *w, &br)) return false;
+    DepGroup::Wait *wt = nullptr;
+    for (auto &q : y.waits)
+        if (q.producer == xi) wt = &q;
+    if (!wt) {
+        y.waits.push_back({xi, std::vector<std::pair<int, int>>((size_t)y.n_tasks, {0, -1})});
+        wt = &y.waits.back();
+    }
+    for (int t = 0; t < y.n_tasks; ++t) {
+        int64_t r0, r1;
+        r->span(t, r0, r1);
+        r0 = std::max<int64_t>(0, r0 + shift);
+        r1 = std::min<int64_t>(w->rows, r1 + shift);
+        if (r1 <= r0) continue;
+        auto &s = wt->span[(size_t)t];
+        const int lo = (int)(r0 / br), hi = (int)((r1 - 1) / br);
+        if (s.second < s.first) s = {lo, hi};
+        else s = {std::min(s.first, lo), std::max(s.second, hi)};
+    }
+    return true;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
 // executor object
 // ---------------------------------------------------------------------------
 struct Executor {
@@ -845,6 +1089,11 @@ struct Executor {
     int grid = 1, threads = 64, lds_bytes = 0;
     int barriers_elided = 0;
     int barriers_local = 0;       // grid barriers replaced by a workgroup-local sync
+    int barriers_counted = 0;     // grid barriers replaced by waits on dependency counters
+    DevWait *d_waits = nullptr;
+    int32_t *d_spans = nullptr, *d_signal = nullptr;
+    unsigned int *d_dep_counters = nullptr;
+    size_t dep_counter_bytes = 0;
     int iteration_sync = 2;       // between iterations of one command: 2 grid barrier, 1 local sync, 0 nothing
     int families = 0;             // OpFamily bits of the compiled ops
     int kernel_families = 0;      // the loop-kernel variant in use
@@ -1055,9 +1304,6 @@ struct Executor {
                 g.signal_begin = -1;
                 const Json &ti = task_infos.at((size_t)st.task_info);
                 const Json &ops_json = ti.at("Ops");
-                if (ops_json.size() > 1 && (st.n_slots != 1 || st.slot_warps != block_warps))
-                    ARK_ERR(UnsupportedError,
-                            "a task with several ops needs one slot spanning the whole workgroup");
                 if (ops_json.size() > 16)
                     ARK_ERR(UnsupportedError, "a task may hold at most 16 ops, got ", ops_json.size());
                 // the ops of one task run for the same task ids: their task counts must agree
@@ -1116,6 +1362,133 @@ struct Executor {
             steps.push_back(ds);
         }
         num_dev_steps = (int)steps.size();
+
+        // ---- dependency counters in place of full-grid barriers --------------------------------
+        // Task groups since the last barrier that stays form a window.  A full-grid barrier inside
+        // the window is replaced by a workgroup sync when every hazard between a group behind it
+        // and a group of the window ahead of it is either local to a workgroup (as above) or a
+        // read of rows whose writers signal counters the reader waits on.  A hazard that is
+        // neither keeps the last barrier ahead of the reader.  ARKMI_DEP_COUNTERS=0 keeps every
+        // barrier.
+        barriers_counted = 0;
+        std::vector<DevWait> h_waits;
+        std::vector<int32_t> h_spans, h_signal;
+        size_t n_counters = 0;
+        {
+            const char *dep_env = getenv("ARKMI_DEP_COUNTERS");
+            bool use_deps = elide && !(dep_env && atoi(dep_env) == 0);
+            for (const auto &st : sched.steps)
+                if (st.is_barrier && !(st.b == 0 && st.e >= grid)) use_deps = false;
+            std::vector<DepGroup> dg;
+            std::vector<int> dg_of_step(sched.steps.size(), -1);
+            if (use_deps) {
+                int segment = 0;
+                for (size_t si = 0; si < sched.steps.size(); ++si) {
+                    if (sched.steps[si].is_barrier) {
+                        ++segment;
+                        continue;
+                    }
+                    DepGroup d;
+                    d.sched_step = (int)si;
+                    d.segment = segment;
+                    d.group = steps[(size_t)dev_step_of[si]].index;
+                    const DevTaskGroup &g = h_groups[(size_t)d.group];
+                    d.n_tasks = std::max(0, (g.task_e - g.task_b + g.task_s - 1) / g.task_s);
+                    d.n_signal = d.n_tasks;
+                    const DevOp &first = ops[(size_t)g.op_begin];
+                    if (first.kind == DEV_GEMM && first.gemm.split_k == 2)
+                        d.n_signal = first.gemm.tiles_m * first.gemm.tiles_n * first.gemm.batch_total;
+                    d.whole_block = g.n_slots == 1 && g.slot_warps == block_warps && g.task_b == 0 && g.task_s == 1;
+                    d.acc = step_accesses(si);
+                    for (int o = g.op_begin; o < g.op_begin + g.op_count; ++o) {
+                        auto r = row_accesses(ops[(size_t)o], g.slot_warps);
+                        d.rows.insert(d.rows.end(), r.begin(), r.end());
+                    }
+                    dg_of_step[si] = (int)dg.size();
+                    dg.push_back(std::move(d));
+                }
+                std::vector<int> window;         // groups since the last barrier that stays
+                std::vector<size_t> candidates;  // full-grid barriers inside the window
+                std::vector<size_t> dropped;
+                for (size_t si = 0; si < sched.steps.size(); ++si) {
+                    if (sched.steps[si].is_barrier) {
+                        if (dev_step_of[si] >= 0 && steps[(size_t)dev_step_of[si]].kind == STEP_BARRIER)
+                            candidates.push_back(si);
+                        continue;
+                    }
+                    const int yi = dg_of_step[si];
+                    int uncovered_after = -1;
+                    for (int xi : window) {
+                        if (dg[(size_t)xi].segment == dg[(size_t)yi].segment) continue;
+                        // (copies: cover_with_counters grows dg[yi].waits, not the access lists)
+                        for (size_t ia = 0; ia < dg[(size_t)xi].acc.size(); ++ia)
+                            for (size_t ib = 0; ib < dg[(size_t)yi].acc.size(); ++ib) {
+                                const Access &ax = dg[(size_t)xi].acc[ia], &ay = dg[(size_t)yi].acc[ib];
+                                if (!overlap(ax, ay) || local_pair(ax, ay)) continue;
+                                if (cover_with_counters(dg, xi, ax, yi, ay, arena, buffer_offset)) continue;
+                                if (getenv("ARKMI_DEBUG_BARRIERS"))
+                                    fprintf(stderr, "no counters for steps %d -> %d: views '%s' (%s) vs '%s' (%s)\n",
+                                            ax.step, ay.step, ax.view.c_str(), ax.write ? "write" : "read",
+                                            ay.view.c_str(), ay.write ? "write" : "read");
+                                uncovered_after = std::max(uncovered_after, dg[(size_t)xi].sched_step);
+                            }
+                    }
+                    if (uncovered_after >= 0) {
+                        // the last barrier ahead of this group stays; what lies between it and the
+                        // group is local to the group's workgroups (judged above), so it waits
+                        // for nothing
+                        if (candidates.empty() || (int)candidates.back() < uncovered_after)
+                            ARK_ERR(InternalError, "no barrier left between steps ", uncovered_after, " and ", si);
+                        const size_t keep = candidates.back();
+                        candidates.pop_back();
+                        dropped.insert(dropped.end(), candidates.begin(), candidates.end());
+                        candidates.clear();
+                        dg[(size_t)yi].waits.clear();
+                        std::vector<int> rest;
+                        for (int xi : window)
+                            if ((size_t)dg[(size_t)xi].sched_step > keep) rest.push_back(xi);
+                        window.swap(rest);
+                    }
+                    window.push_back(yi);
+                }
+                dropped.insert(dropped.end(), candidates.begin(), candidates.end());
+                // a barrier behind the last group orders nothing inside the body: it is not counted
+                for (size_t si : dropped) {
+                    steps[(size_t)dev_step_of[si]].kind = STEP_LOCAL_SYNC;
+                    ++barriers_counted;
+                }
+            }
+            if (barriers_counted > 0) {
+                for (auto &y : dg)
+                    for (auto &w : y.waits) {
+                        DepGroup &x = dg[(size_t)w.producer];
+                        if (x.counter_base < 0) {
+                            x.counter_base = (int)n_counters;
+                            n_counters += (size_t)x.n_blocks;
+                        }
+                    }
+                for (auto &d : dg) {
+                    DevTaskGroup &g = h_groups[(size_t)d.group];
+                    if (d.counter_base >= 0) {
+                        g.signal_begin = (int)h_signal.size();
+                        g.signal_base = d.counter_base;
+                        h_signal.insert(h_signal.end(), d.signal_map.begin(), d.signal_map.end());
+                    }
+                    if (!d.waits.empty()) {
+                        g.n_waits = (int)d.waits.size();
+                        g.wait_begin = (int)h_waits.size();
+                        g.span_begin = (int)h_spans.size();
+                        for (const auto &w : d.waits)
+                            h_waits.push_back(DevWait{dg[(size_t)w.producer].counter_base, dg[(size_t)w.producer].per_block});
+                        for (int t = 0; t < d.n_tasks; ++t)
+                            for (const auto &w : d.waits) {
+                                h_spans.push_back(w.span[(size_t)t].first);
+                                h_spans.push_back(w.span[(size_t)t].second);
+                            }
+                    }
+                }
+            }
+        }
 
         // The boundary between two iterations of one command is one more barrier
         // candidate: what runs after the body's last full barrier meets what runs
@@ -1178,6 +1551,9 @@ struct Executor {
             const char *it_env = getenv("ARKMI_ITERATION_BARRIER");
             if (it_env ? atoi(it_env) != 0 : (families & (FAM_GEMM | FAM_ATTN)) == 0) iteration_sync = 2;
         }
+        // the counters count per iteration, and a reader relies on the caches having been
+        // invalidated since the previous one
+        if (barriers_counted > 0) iteration_sync = 2;
         lds_bytes = loop_kernel_lds_reserved() + max_slot_lds;
         const auto &facts = device_facts(device);
         if (lds_bytes > facts.lds_bytes)
@@ -1205,6 +1581,18 @@ struct Executor {
             ARKMI_HIP(hipMalloc((void **)&d_trace, trace_len * sizeof(TraceRecord)));
             ARKMI_HIP(hipMemset(d_trace, 0xff, trace_len * sizeof(TraceRecord)));
         }
+        if (barriers_counted > 0) {
+            upload(h_waits.data(), h_waits.size() * sizeof(DevWait), (void **)&d_waits);
+            upload(h_spans.data(), h_spans.size() * sizeof(int32_t), (void **)&d_spans);
+            upload(h_signal.data(), h_signal.size() * sizeof(int32_t), (void **)&d_signal);
+            dep_counter_bytes = n_counters * kDepStride * sizeof(unsigned int);
+            ARKMI_HIP(hipMalloc((void **)&d_dep_counters, dep_counter_bytes));
+            ARKMI_HIP(hipMemset(d_dep_counters, 0, dep_counter_bytes));
+        }
+        prog.waits = d_waits;
+        prog.wait_spans = d_spans;
+        prog.signal_map = d_signal;
+        prog.dep_counters = d_dep_counters;
         prog.steps = d_steps;
         prog.groups = d_groups;
         prog.ops = d_ops;
@@ -1235,6 +1623,7 @@ struct Executor {
     void start_kernel() {
         // control block and mailbox start from zero on every kernel launch
         ARKMI_HIP(hipMemsetAsync(ctl, 0, sizeof(LoopControl), stream));
+        if (d_dep_counters) ARKMI_HIP(hipMemsetAsync(d_dep_counters, 0, dep_counter_bytes, stream));
         mb->status = MB_OK;
         mb->alive = 1;
         loop_kernel_launch(kernel, prog, ctl, mb_dev, grid, threads, lds_bytes, 0, idle_ticks, wait_ticks, stream);
@@ -1275,6 +1664,7 @@ struct Executor {
             __atomic_store_n(&mb->cmd, iter, __ATOMIC_RELEASE);
         } else {
             ARKMI_HIP(hipMemsetAsync(ctl, 0, sizeof(LoopControl), stream));
+            if (d_dep_counters) ARKMI_HIP(hipMemsetAsync(d_dep_counters, 0, dep_counter_bytes, stream));
             loop_kernel_launch(kernel, prog, ctl, mb_dev, grid, threads, lds_bytes, iter, idle_ticks, wait_ticks,
                                stream);
         }
@@ -1368,7 +1758,8 @@ struct Executor {
         }
         (void)hipSetDevice(device);
         for (void *p : {(void *)arena, (void *)ctl, (void *)d_ops, (void *)d_groups, (void *)d_steps,
-                        (void *)d_trace, (void *)d_clock})
+                        (void *)d_trace, (void *)d_clock, (void *)d_waits, (void *)d_spans, (void *)d_signal,
+                        (void *)d_dep_counters})
             if (p) (void)hipFree(p);
         for (void *p : scratch_allocs) (void)hipFree(p);
         scratch_allocs.clear();
@@ -1377,7 +1768,8 @@ struct Executor {
         if (ev_end) (void)hipEventDestroy(ev_end);
         if (own_stream && stream) (void)hipStreamDestroy(stream);
         arena = nullptr; ctl = nullptr; d_ops = nullptr; d_groups = nullptr; d_steps = nullptr;
-        d_trace = nullptr; d_clock = nullptr; mb = nullptr; ev_begin = ev_end = nullptr; stream = nullptr;
+        d_trace = nullptr; d_clock = nullptr; d_waits = nullptr; d_spans = nullptr; d_signal = nullptr;
+        d_dep_counters = nullptr; mb = nullptr; ev_begin = ev_end = nullptr; stream = nullptr;
         destroyed = true;
     }
 
@@ -1588,6 +1980,7 @@ int arkmi_exec_info(arkmi_exec *h, arkmi_exec_info_t *out) {
         out->iterations_done = h->ex.mb ? h->ex.mb->done : 0;
         out->barriers_local = h->ex.barriers_local;
         out->iteration_sync = h->ex.iteration_sync;
+        out->barriers_counted = h->ex.barriers_counted;
     });
 }
 

@@ -137,8 +137,14 @@ __device__ __forceinline__ void drain_stores_then_barrier() {
 // ---- slot context -----------------------------------------------------------
 // A task runs on one "slot": a contiguous group of waves of the workgroup with
 // its own LDS window.  With one resident slot per CU (the gfx950 default) the
-// slot is the whole workgroup and sync() is a plain s_barrier.
+// slot is the whole workgroup and sync() is a plain s_barrier.  A plan may run
+// several narrower slots side by side (tasks of fewer warps than the workgroup
+// has); their waves then meet on a counter in LDS, one per slot, as the
+// reference does on this architecture (ark/include/kernels/common/sync.h:108-127).
 using lds_ptr = __attribute__((address_space(3))) char *;
+using lds_u32_ptr = __attribute__((address_space(3))) unsigned int *;
+
+constexpr unsigned kSlotSyncSpinLimit = 1u << 26;  // polls before a slot barrier gives up waiting
 
 struct Slot {
     int tid;        // thread index inside the slot
@@ -146,13 +152,36 @@ struct Slot {
     lds_ptr lds;    // slot's LDS window
     int lds_bytes;  // bytes in the window
     bool whole_block;
+    // The slot's arrival counter (null for a slot that spans the workgroup).  It only
+    // grows: with W waves per slot, barrier number g is complete when it reaches g * W.
+    lds_u32_ptr arrivals = nullptr;
     __device__ __forceinline__ int lane() const { return tid & 63; }
     __device__ __forceinline__ int wave() const { return tid >> 6; }
     __device__ __forceinline__ int nwaves() const { return nthreads >> 6; }
     __device__ __forceinline__ void sync() const {
-        // Sub-block slots are rejected on the host until a partial barrier is
-        // implemented; every slot seen here spans the workgroup.
-        __syncthreads();
+        if (whole_block || arrivals == nullptr) {
+            __syncthreads();
+            return;
+        }
+        if (nthreads <= 64) {  // one wave: nothing to meet, only this wave's own memory order
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+            __builtin_amdgcn_wave_barrier();
+            return;
+        }
+        // this wave's LDS and global traffic is complete before it counts as arrived
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        if (lane() == 0) {
+            const unsigned w = (unsigned)nwaves();
+            const unsigned old = __hip_atomic_fetch_add(arrivals, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const unsigned target = (old / w + 1u) * w;
+            unsigned spins = 0;
+            while ((int)(__hip_atomic_load(arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) - target) < 0) {
+                __builtin_amdgcn_s_sleep(1);
+                if (++spins > kSlotSyncSpinLimit) break;  // never hang the CU
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+        __builtin_amdgcn_wave_barrier();
     }
 };
 

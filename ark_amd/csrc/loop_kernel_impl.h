@@ -243,106 +243,113 @@ __device__ __forceinline__ D load_karg(const ARKMI_CONST D *p) {
 #define KARG(field) load_karg(&kargs()->field)
 
 // ---- the long-running bodies -----------------------------------------------------------------
+#ifndef ARKMI_BODY
 #define ARKMI_BODY __device__ __attribute__((noinline))
+#endif
 
-// A long-running op owns the whole workgroup (checked on the host): its slot is the first one.
-__device__ __forceinline__ Slot body_slot(int tid) {
+// What a body receives: the address of its op descriptor, the task, the thread index and the
+// address of the workgroup's LDS window (a long-running op owns the whole workgroup, checked on
+// the host).  All but the thread index are uniform and are moved to scalar registers here.  A
+// body must not use the kernel-argument segment: its address is not passed on to a function.
+__device__ __forceinline__ const DevOp *uniform_op(const DevOp *op) {
+    const uint64_t a = reinterpret_cast<uint64_t>(op);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    return reinterpret_cast<const DevOp *>(((uint64_t)hi << 32) | lo);
+}
+
+__device__ __forceinline__ Slot body_slot(int tid, lds_ptr lds) {
     Slot s;
     s.tid = tid;
-    s.nthreads = blockDim.x;
-    s.lds = (lds_ptr)g_loop_lds + kLdsReserved;
+    s.nthreads = kLoopMaxThreads;  // (not read by these bodies)
+    s.lds = (lds_ptr)(uintptr_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
     s.lds_bytes = 0;
     s.whole_block = true;
     return s;
 }
 
-__device__ __forceinline__ const DevOp *body_op(int op_index) {
-    return KARG(prog.ops) + __builtin_amdgcn_readfirstlane(op_index);
-}
-
 // One matmul tile shape.  Returns the task index the ops fused behind the matmul run for (the
 // tile this workgroup finished), -1 when another workgroup finishes the tile (a split of K).
 template <typename T, int BM, int BN, bool TRANS_B, bool TRANS_A = false, bool DUAL_B = false, bool SPLIT = false>
-ARKMI_BODY int gemm_body(int op_index, int task, int tid) {
-    const GemmDesc g = load_const(&body_op(op_index)->gemm);
+ARKMI_BODY int gemm_body(const DevOp *op, int task, int tid, lds_ptr lds) {
+    const GemmDesc g = load_const(&uniform_op(op)->gemm);
     return gemm_tile<T, BM, BN, TRANS_B, EpilogueStore, TRANS_A, DUAL_B, SPLIT>(
-        g, __builtin_amdgcn_readfirstlane(task), body_slot(tid), EpilogueStore());
+        g, __builtin_amdgcn_readfirstlane(task), body_slot(tid, lds), EpilogueStore());
 }
 
-ARKMI_BODY int gemm_f32_body(int op_index, int task, int tid) {
-    const GemmDesc g = load_const(&body_op(op_index)->gemm);
-    gemm_f32_dispatch(g, __builtin_amdgcn_readfirstlane(task), body_slot(tid));
+ARKMI_BODY int gemm_f32_body(const DevOp *op, int task, int tid, lds_ptr lds) {
+    const GemmDesc g = load_const(&uniform_op(op)->gemm);
+    gemm_f32_dispatch(g, __builtin_amdgcn_readfirstlane(task), body_slot(tid, lds));
     return task;
 }
 
-ARKMI_BODY int gemv_body(int op_index, int task, int tid) {
-    const GemvDesc d = load_const(&body_op(op_index)->gemv);
-    gemv_dispatch(d, __builtin_amdgcn_readfirstlane(task), body_slot(tid));
+ARKMI_BODY int gemv_body(const DevOp *op, int task, int tid, lds_ptr lds) {
+    const GemvDesc d = load_const(&uniform_op(op)->gemv);
+    gemv_dispatch(d, __builtin_amdgcn_readfirstlane(task), body_slot(tid, lds));
     return task;
 }
 
-ARKMI_BODY int attn_body(int op_index, int task, int tid) {
-    const AttnDesc d = load_const(&body_op(op_index)->attn);
-    attn_dispatch(d, __builtin_amdgcn_readfirstlane(task), body_slot(tid));
+ARKMI_BODY int attn_body(const DevOp *op, int task, int tid, lds_ptr lds) {
+    const AttnDesc d = load_const(&uniform_op(op)->attn);
+    attn_dispatch(d, __builtin_amdgcn_readfirstlane(task), body_slot(tid, lds));
     return task;
 }
 
 template <int FAM, typename T, bool TRANS_B>
-__device__ __forceinline__ int gemm_by_tile(const DevOp *op, int op_index, int task, int tid) {
+__device__ __forceinline__ int gemm_by_tile(const DevOp *op, int task, int tid, lds_ptr lds) {
     const int tm = load_const(&op->gemm_tile_m), tn = load_const(&op->gemm_tile_n);
     if (load_const(&op->gemm.split_k) == 2) {  // 256x256 tiles only (checked on the host)
         if constexpr ((FAM & FAM_SPLITK) != 0)
-            return gemm_body<T, 256, 256, TRANS_B, false, false, true>(op_index, task, tid);
+            return gemm_body<T, 256, 256, TRANS_B, false, false, true>(op, task, tid, lds);
         else
             return -1;
     }
     if constexpr (TRANS_B) {
         if (load_const(&op->gemm.b2) != nullptr) {  // gate/up pair: 256-wide tiles only (checked on the host)
-            if (tm == 256) return gemm_body<T, 256, 256, true, false, true>(op_index, task, tid);
-            return gemm_body<T, 128, 256, true, false, true>(op_index, task, tid);
+            if (tm == 256) return gemm_body<T, 256, 256, true, false, true>(op, task, tid, lds);
+            return gemm_body<T, 128, 256, true, false, true>(op, task, tid, lds);
         }
     }
-    if (tm == 256 && tn == 256) return gemm_body<T, 256, 256, TRANS_B>(op_index, task, tid);
-    if (tm == 128 && tn == 256) return gemm_body<T, 128, 256, TRANS_B>(op_index, task, tid);
-    if (tm == 256 && tn == 128) return gemm_body<T, 256, 128, TRANS_B>(op_index, task, tid);
-    return gemm_body<T, 128, 128, TRANS_B>(op_index, task, tid);
+    if (tm == 256 && tn == 256) return gemm_body<T, 256, 256, TRANS_B>(op, task, tid, lds);
+    if (tm == 128 && tn == 256) return gemm_body<T, 128, 256, TRANS_B>(op, task, tid, lds);
+    if (tm == 256 && tn == 128) return gemm_body<T, 256, 128, TRANS_B>(op, task, tid, lds);
+    return gemm_body<T, 128, 128, TRANS_B>(op, task, tid, lds);
 }
 
 // The first op of a task, of the long-running kind KIND, for one task.  Returns (uniformly) the
 // task index for the ops that follow in the same fused task: `task` itself, except behind a
 // matmul that splits K, where it is the tile this workgroup finished or -1 (none).
 template <int FAM, int KIND>
-__device__ __forceinline__ int run_long(int op_index, int task, int tid) {
-    const DevOp *op = KARG(prog.ops) + op_index;
+__device__ __forceinline__ int run_long(const DevOp *op, int task, int tid, lds_ptr lds) {
     int follow = task;
     if constexpr (KIND == DEV_GEMM) {
         const int dtype = load_const(&op->gemm.dtype);
         const bool trans_a = load_const(&op->gemm.trans_a) != 0, trans_b = load_const(&op->gemm.trans_b) != 0;
         if (dtype == 0 || trans_a) {
             if constexpr ((FAM & FAM_EXT) != 0) {
-                if (dtype == 0) gemm_f32_body(op_index, task, tid);
+                if (dtype == 0) gemm_f32_body(op, task, tid, lds);
                 else if (dtype == 1) {
-                    if (trans_b) gemm_body<f16, 128, 128, true, true>(op_index, task, tid);
-                    else gemm_body<f16, 128, 128, false, true>(op_index, task, tid);
+                    if (trans_b) gemm_body<f16, 128, 128, true, true>(op, task, tid, lds);
+                    else gemm_body<f16, 128, 128, false, true>(op, task, tid, lds);
                 } else {
-                    if (trans_b) gemm_body<bf16, 128, 128, true, true>(op_index, task, tid);
-                    else gemm_body<bf16, 128, 128, false, true>(op_index, task, tid);
+                    if (trans_b) gemm_body<bf16, 128, 128, true, true>(op, task, tid, lds);
+                    else gemm_body<bf16, 128, 128, false, true>(op, task, tid, lds);
                 }
             }
         } else if constexpr ((FAM & FAM_GEMM) != 0) {
             if (dtype == 1) {
-                follow = trans_b ? gemm_by_tile<FAM, f16, true>(op, op_index, task, tid)
-                                 : gemm_by_tile<FAM, f16, false>(op, op_index, task, tid);
+                follow = trans_b ? gemm_by_tile<FAM, f16, true>(op, task, tid, lds)
+                                 : gemm_by_tile<FAM, f16, false>(op, task, tid, lds);
             } else {
-                follow = trans_b ? gemm_by_tile<FAM, bf16, true>(op, op_index, task, tid)
-                                 : gemm_by_tile<FAM, bf16, false>(op, op_index, task, tid);
+                follow = trans_b ? gemm_by_tile<FAM, bf16, true>(op, task, tid, lds)
+                                 : gemm_by_tile<FAM, bf16, false>(op, task, tid, lds);
             }
             follow = __builtin_amdgcn_readfirstlane(follow);
         }
     } else if constexpr (KIND == DEV_GEMV) {
-        if constexpr ((FAM & FAM_GEMV) != 0) gemv_body(op_index, task, tid);
+        if constexpr ((FAM & FAM_GEMV) != 0) gemv_body(op, task, tid, lds);
     } else if constexpr (KIND == DEV_ATTN) {
-        if constexpr ((FAM & FAM_ATTN) != 0) attn_body(op_index, task, tid);
+        if constexpr ((FAM & FAM_ATTN) != 0) attn_body(op, task, tid, lds);
     }
     return follow;
 }
@@ -356,9 +363,9 @@ struct TaskDeal {
     bool mine;      // this workgroup is in the group's processor range
 };
 
-__device__ __forceinline__ TaskDeal deal_of(int gi) {
+__device__ __forceinline__ TaskDeal deal_of(const DevTaskGroup *groups, int gi) {
     TaskDeal d;
-    d.g = load_const(KARG(prog.groups) + gi);
+    d.g = load_const(groups + gi);
     const DevTaskGroup &g = d.g;
     const int block = blockIdx.x, grid = gridDim.x;
     d.mine = in_range(block, g.proc_b, g.proc_e, g.proc_s);
@@ -427,23 +434,30 @@ __device__ __forceinline__ void trace_task(const DevTaskGroup &g, int64_t id, in
 #endif
 }
 
-// The task loop of a group of small ops: the group's parameters stay in registers.
+// The task loop of a group of small ops: the program's and the group's parameters stay in
+// registers (`P` was read once for the step).
 template <int FAM>
-__device__ __forceinline__ bool run_small_tasks(int gi, const TaskDeal &d, const Slot &s, int slot_k, unsigned epoch) {
+__device__ __forceinline__ bool run_small_tasks(const LoopProgram &P, const TaskDeal &d, const Slot &s, int slot_k,
+                                                unsigned epoch) {
     const DevTaskGroup &g = d.g;
-    const DevOp *ops = KARG(prog.ops) + g.op_begin;
-    const bool deps = KARG(prog.dep_counters) != nullptr;
+    const DevOp *ops = P.ops + g.op_begin;
+    const bool deps = P.dep_counters != nullptr;
     const bool waits = deps && g.n_waits > 0, signals = deps && g.signal_begin >= 0;
     int order = 0;
     for (unsigned t = (unsigned)slot_k;; t += (unsigned)g.n_slots, ++order) {
         const int64_t id = task_id(d, t);
         if (id >= g.task_e) break;
         const int ti = (waits || signals) ? task_index(g, id) : 0;
-        trace_task(g, id, slot_k, order, s);
+#ifndef ARKMI_NO_TRACE
+        if (P.trace && g.trace_offset >= 0 && s.tid == 0) {
+            TraceRecord rec{(int)blockIdx.x, slot_k, order};
+            P.trace[g.trace_offset + task_index(g, id)] = rec;
+        }
+#endif
         if (waits && !wait_for_rows(g, ti, s, epoch)) return false;
         for (int o = 0; o < g.op_count; ++o) {
-            // later ops of a fused task read what earlier ones of the same workgroup wrote:
-            // the workgroup meets (its waves share one L1, which sees their stores)
+            // later ops of a fused task read what earlier ones of the same slot wrote: the slot's
+            // waves meet (they share one L1, which sees their stores)
             if (o > 0) s.sync();
             run_small<FAM>(ops + o, (int)id, s);
         }
@@ -462,14 +476,14 @@ __device__ __forceinline__ bool run_long_tasks(int gi, const Slot &s, int slot_k
     for (unsigned t = (unsigned)slot_k;; ++order) {
         int follow;
         {
-            const TaskDeal d = deal_of(gi);
+            const TaskDeal d = deal_of(KARG(prog.groups), gi);
             const DevTaskGroup &g = d.g;
             const int64_t id = task_id(d, t);
             if (id >= g.task_e) break;
             const bool deps = KARG(prog.dep_counters) != nullptr;
             trace_task(g, id, slot_k, order, s);
             if (deps && g.n_waits > 0 && !wait_for_rows(g, task_index(g, id), s, epoch)) return false;
-            follow = run_long<FAM, KIND>(g.op_begin, (int)id, s.tid);  // uniform across the workgroup
+            follow = run_long<FAM, KIND>(KARG(prog.ops) + g.op_begin, (int)id, s.tid, s.lds);  // uniform across the workgroup
         }
         const DevTaskGroup g = load_const(KARG(prog.groups) + gi);
         if constexpr (KIND == DEV_GEMM) {
@@ -487,9 +501,16 @@ __device__ __forceinline__ bool run_long_tasks(int gi, const Slot &s, int slot_k
     return true;
 }
 
+// Does this variant hold a long-running body?  If not, nothing competes for scalar registers
+// and the program's parameters are read once per launch instead of once per step.
 template <int FAM>
-__device__ __forceinline__ bool run_group(int gi, unsigned epoch) {
-    const TaskDeal d = deal_of(gi);
+constexpr bool kHasLongBodies = (FAM & (FAM_GEMM | FAM_SPLITK | FAM_EXT | FAM_GEMV | FAM_ATTN)) != 0;
+
+constexpr int kLdsSlotCounters = 64;  // byte offset of the slots' arrival counters in the control area
+
+template <int FAM>
+__device__ __forceinline__ bool run_group(const LoopProgram &P, int gi, unsigned epoch) {
+    const TaskDeal d = deal_of(P.groups, gi);
     const DevTaskGroup &g = d.g;
     if (!d.mine) return true;
     const int slot_threads = g.slot_warps * kWave;
@@ -501,9 +522,10 @@ __device__ __forceinline__ bool run_group(int gi, unsigned epoch) {
     s.lds = (lds_ptr)g_loop_lds + kLdsReserved + k * g.slot_sram;
     s.lds_bytes = g.slot_sram;
     s.whole_block = (slot_threads == (int)blockDim.x);
+    s.arrivals = s.whole_block ? nullptr : (lds_u32_ptr)((lds_ptr)g_loop_lds + kLdsSlotCounters) + k;
     // one task loop per long-running kind of first op, one for the tasks of small ops
     // (a variant holds the loops of the families it was built for)
-    const int first = load_const(&(KARG(prog.ops) + g.op_begin)->kind);
+    const int first = load_const(&(P.ops + g.op_begin)->kind);
     if constexpr ((FAM & (FAM_GEMM | FAM_SPLITK | FAM_EXT)) != 0) {
         if (first == DEV_GEMM) return run_long_tasks<FAM, DEV_GEMM>(gi, s, k, epoch);
     }
@@ -515,18 +537,28 @@ __device__ __forceinline__ bool run_group(int gi, unsigned epoch) {
     }
     if constexpr ((FAM & (FAM_ROW | FAM_EWISE | FAM_EXT)) != 0) {
         if (first != DEV_GEMM && first != DEV_GEMV && first != DEV_ATTN)
-            return run_small_tasks<FAM>(gi, d, s, k, epoch);
+            return run_small_tasks<FAM>(P, d, s, k, epoch);
     }
     return true;
 }
 
+// The control words at the start of the workgroup's LDS: [0] the barriers' verdict, [1] raised
+// when a dependency wait gave up, from byte kLdsSlotCounters one arrival counter per slot.
+__device__ __forceinline__ void init_lds_control() {
+    if (threadIdx.x == 0) reinterpret_cast<volatile int *>(g_loop_lds)[1] = 0;
+    if (threadIdx.x < 8) reinterpret_cast<volatile unsigned *>(g_loop_lds + kLdsSlotCounters)[threadIdx.x] = 0u;
+    __syncthreads();
+}
+
 // One iteration of the plan's body; `epoch` counts the iterations since the launch from 1.
 template <int FAM>
-__device__ __forceinline__ bool run_body(XcdInfo &xi, unsigned epoch) {
-    for (int si = 0; si < KARG(prog.num_steps); ++si) {
-        const DevStep st = load_const(KARG(prog.steps) + si);
-        unsigned long long *clock = KARG(prog.step_clock);
-        if (clock && threadIdx.x == 0) clock[(size_t)blockIdx.x * (KARG(prog.num_steps) + 1) + si] = wall_clock64();
+__device__ __forceinline__ bool run_body(const LoopProgram &P0, XcdInfo &xi, unsigned epoch) {
+    const int num_steps = kHasLongBodies<FAM> ? KARG(prog.num_steps) : P0.num_steps;
+    for (int si = 0; si < num_steps; ++si) {
+        // (one read of the whole parameter block per step where long bodies want the registers)
+        const LoopProgram P = kHasLongBodies<FAM> ? KARG(prog) : P0;
+        const DevStep st = load_const(P.steps + si);
+        if (P.step_clock && threadIdx.x == 0) P.step_clock[(size_t)blockIdx.x * (P.num_steps + 1) + si] = wall_clock64();
         if (st.kind == STEP_BARRIER) {
             LoopControl *ctl = KARG(ctl);
             if ((unsigned)st.count == gridDim.x) {
@@ -539,14 +571,11 @@ __device__ __forceinline__ bool run_body(XcdInfo &xi, unsigned epoch) {
             // L1, which sees their own stores, so the workgroup only has to meet
             __syncthreads();
         } else {
-            if (!run_group<FAM>(st.index, epoch)) return false;
+            if (!run_group<FAM>(P, st.index, epoch)) return false;
         }
     }
     unsigned long long *clock = KARG(prog.step_clock);
-    if (clock && threadIdx.x == 0) {
-        const int n = KARG(prog.num_steps);
-        clock[(size_t)blockIdx.x * (n + 1) + n] = wall_clock64();
-    }
+    if (clock && threadIdx.x == 0) clock[(size_t)blockIdx.x * (num_steps + 1) + num_steps] = wall_clock64();
     return true;
 }
 
@@ -554,8 +583,7 @@ template <int FAM>
 __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(LoopArgs) {
     const unsigned nblocks = gridDim.x;
     const bool leader = (blockIdx.x == 0 && threadIdx.x == 0);
-    // LDS control words: [0] the barriers' verdict, [1] raised when a dependency wait gave up
-    if (threadIdx.x == 0) reinterpret_cast<volatile int *>(g_loop_lds)[1] = 0;
+    init_lds_control();
     // count the workgroups per XCD (the control block is zeroed before every launch)
     XcdInfo xi;
     xi.epoch = 0;
@@ -577,6 +605,7 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(LoopArgs) {
             xi.nxcd += __hip_atomic_load(&ctl->xcd_blocks[i], __ATOMIC_RELAXED, AGENT) ? 1u : 0u;
     }
     unsigned epoch = 0;  // iterations of the body started since the launch
+    const LoopProgram P0 = KARG(prog);
     for (;;) {
         int iter;
         const int one_shot_iters = KARG(one_shot_iters);
@@ -624,7 +653,7 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(LoopArgs) {
                 }
             }
             ++epoch;
-            if (ok) ok = run_body<FAM>(xi, epoch);
+            if (ok) ok = run_body<FAM>(P0, xi, epoch);
         }
         if (!ok) break;
         // results must be visible to the host before the command is cleared: every
@@ -653,8 +682,9 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(LoopArgs) {
 // boundaries order everything.
 template <int FAM>
 __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_step_kernel(LoopArgs) {
-    if (threadIdx.x == 0) reinterpret_cast<volatile int *>(g_loop_lds)[1] = 0;
-    run_group<FAM>(KARG(group), 1u);
+    init_lds_control();
+    const LoopProgram P = KARG(prog);
+    run_group<FAM>(P, KARG(group), 1u);
 }
 
 // Defines the host-visible handles of one kernel variant; each variant is its own

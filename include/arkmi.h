@@ -50,6 +50,11 @@ enum arkmi_dtype {
 const char *arkmi_last_error(void);
 const char *arkmi_version(void);
 
+/* ark::init() (ark/api/init.cpp:15-19): reads the ARK_* environment variables again
+ * (ARK_LOG_LEVEL, ARK_ENFORCE_PLAN_PATH, ...); they are otherwise read once, on first use.
+ * This backend keeps no temporary directory, so there is nothing else to set up. */
+int arkmi_init(void);
+
 /* Device facts the planner reads (ark/gpu/gpu_manager.cpp:29-75: num_sm, arch
  * name, max threads/LDS).  arch is written as "ROCM_950" style text. */
 typedef struct arkmi_device_info {
@@ -256,6 +261,7 @@ typedef struct arkmi_exec_info_t {
     int iterations_done;
     int barriers_local;   /* grid barriers replaced by a workgroup-local sync */
     int iteration_sync;   /* between iterations of one run(n): 2 grid barrier, 1 workgroup-local sync, 0 nothing */
+    int barriers_counted; /* grid barriers replaced by waits on per-row-block dependency counters */
 } arkmi_exec_info_t;
 
 int arkmi_exec_create(int device_id, void *stream, const char *name,

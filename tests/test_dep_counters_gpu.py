@@ -1,0 +1,118 @@
+"""Dependency counters in place of grid barriers (the loop kernel's per-row-block counters in
+device memory): each graph runs with the counters and with every barrier kept
+(ARKMI_DEP_COUNTERS=0); outputs must agree bit for bit over several iterations, in the resident
+loop kernel and in one-shot launches, and the executor must report which barriers it replaced.
+The reference orders the same chains with one sync_gpu per op boundary (ark/codegen.cpp:109-158)."""
+import numpy as np
+import pytest
+
+from helpers import make
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(m, feeds, fetch, iters, loop_mode=True):
+    from ark_amd import Executor
+    ex = Executor(m.plan(device_id=0), device_id=0, loop_mode=loop_mode).compile()
+    for t, a in feeds.items():
+        ex.tensor_write(t, a)
+    ex.launch()
+    ex.run(iters)
+    ex.wait()
+    outs = [ex.tensor_read(t) for t in fetch]
+    info = ex.info()
+    ex.stop()
+    return outs, info
+
+
+def rows_gemm_gemm(m, dt):
+    x, w1, w2 = m.tensor([1024, 1024], dt), m.tensor([1024, 2048], dt), m.tensor([2048, 1024], dt)
+    return [x, w1, w2], [m.matmul(m.matmul(m.rmsnorm(x), w1), w2)], 2
+
+
+def gemm_rows_gemm(m, dt):
+    x, w1, w2 = m.tensor([1024, 512], dt), m.tensor([512, 1024], dt), m.tensor([1024, 512], dt)
+    h = m.matmul(x, w1)
+    return [x, w1, w2], [m.matmul(m.softmax(h), w2), m.reduce_sum(h, -1)], 2
+
+
+def gemm_with_follower_feeds_gemm(m, dt):
+    x, w1, w2, r = (m.tensor([1024, 1024], dt), m.tensor([1024, 1024], dt), m.tensor([1024, 1024], dt),
+                    m.tensor([1024, 1024], dt))
+    with m.planner_context(sync=False):
+        h = m.add(r, m.matmul(x, w1))
+    return [x, w1, w2, r], [m.matmul(h, w2, trans_other=True)], 1
+
+
+def projections_attention_projection(m, dt):
+    seq, heads, hd = 512, 4, 128
+    dim = heads * hd
+    x = m.tensor([1, seq, dim], dt)
+    wq, wk, wv, wo = (m.tensor([dim, dim], dt) for _ in range(4))
+    q = m.reshape(m.matmul(x, wq, trans_other=True), [1, seq, heads, hd])
+    k = m.reshape(m.matmul(x, wk, trans_other=True), [1, seq, heads, hd])
+    v = m.reshape(m.matmul(x, wv, trans_other=True), [1, seq, heads, hd])
+    a = m.reshape(m.attention(q, k, v, hd ** -0.5, causal=True), [1, seq, dim])
+    return [x, wq, wk, wv, wo], [m.matmul(a, wo, trans_other=True)], 2
+
+
+def in_place_residual_loop(m, dt):
+    """x <- x + rmsnorm(x) @ w: every iteration reads what the previous one wrote, so the boundary
+    between iterations keeps its grid barrier.  (At this size the ops run on sub-ranges of the
+    workgroups, whose barriers are never replaced: the graph checks that nothing else changes.)"""
+    x, w = m.tensor([512, 512], dt), m.tensor([512, 512], dt)
+    h = m.matmul(m.rmsnorm(x), w)
+    out = m.add(x, m.mul(h, 0.01), output=x)
+    return [x, w], [out], 0
+
+
+GRAPHS = {f.__name__: f for f in (rows_gemm_gemm, gemm_rows_gemm, gemm_with_follower_feeds_gemm,
+                                  projections_attention_projection, in_place_residual_loop)}
+
+
+@pytest.mark.parametrize("loop_mode", [True, False])
+@pytest.mark.parametrize("graph", sorted(GRAPHS))
+def test_counters_give_the_barriers_results(oracle, graph, loop_mode, monkeypatch):
+    from ark_amd import Model
+    dtype = "bf16" if "attention" in graph else "fp16"
+    results = {}
+    for counters in ("0", "1"):
+        monkeypatch.setenv("ARKMI_DEP_COUNTERS", counters)
+        m = Model()
+        ins, fetch, least = GRAPHS[graph](m, dtype)
+        feeds = {t: make(oracle, tuple(t.shape), dtype, 700 + i, "uniform", -0.5, 0.5) for i, t in enumerate(ins)}
+        outs, info = _run(m, feeds, fetch, iters=4, loop_mode=loop_mode)
+        if counters == "0":
+            assert info["barriers_counted"] == 0
+        else:
+            assert info["barriers_counted"] >= least, info
+            assert least == 0 or info["iteration_sync"] == 2
+        results[counters] = outs
+    for a, b in zip(results["0"], results["1"]):
+        assert np.isfinite(a.astype(np.float32)).all()
+        assert np.array_equal(a, b), graph
+
+
+def test_counters_across_commands_and_relaunch(oracle, monkeypatch):
+    """The counters count iterations since the kernel's launch: several run() commands on one
+    resident kernel, then a stop and a second launch (counters start from zero again)."""
+    from ark_amd import Model, Executor
+    dtype = "fp16"
+    m = Model()
+    ins, fetch, _ = rows_gemm_gemm(m, dtype)
+    feeds = {t: make(oracle, tuple(t.shape), dtype, 800 + i, "uniform", -0.5, 0.5) for i, t in enumerate(ins)}
+    monkeypatch.setenv("ARKMI_DEP_COUNTERS", "0")
+    (want,), _ = _run(m, feeds, fetch, iters=1)
+    monkeypatch.setenv("ARKMI_DEP_COUNTERS", "1")
+    ex = Executor(m.plan(device_id=0), device_id=0).compile()
+    assert ex.info()["barriers_counted"] >= 2
+    for t, a in feeds.items():
+        ex.tensor_write(t, a)
+    for launch in range(2):
+        ex.launch()
+        for n in (1, 3, 2):
+            ex.tensor_write(fetch[0], np.zeros(fetch[0].shape, np.float16))
+            ex.run(n)
+            ex.wait()
+            assert np.array_equal(ex.tensor_read(fetch[0]), want), (launch, n)
+        ex.stop()

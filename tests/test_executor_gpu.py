@@ -960,3 +960,45 @@ def test_grid_barrier_drops_other_workgroups_old_lines_from_the_l1(oracle):
     for _ in range(iters):
         want = np.ascontiguousarray(want.transpose(0, 1, 3, 2)) + np.float32(1.0)
     assert np.array_equal(got, want)
+
+
+# ---------------------------------------------------------------- several slots per workgroup
+def test_fused_task_in_two_warp_slots(oracle):
+    """Tasks of two warps run four to a workgroup, each slot on its own waves; the ops of a fused
+    task then meet on the slot's own barrier (ark/include/kernels/common/sync.h:81-130), not on
+    the workgroup's.  500 tasks over 4 slots x 256 workgroups leaves slots with unequal task
+    counts, so a workgroup-wide barrier inside the task would pair the wrong waves."""
+    from ark_amd import Model
+    dtype = "fp16"
+    m = Model()
+    t0, t1 = m.tensor((4000, 256), dtype), m.tensor((4000, 256), dtype)
+    cfg = {"NumWarps": 2, "SramBytes": 0, "Tile": [8, 256], "NumTasks": 500}
+    with m.planner_context(sync=False, config=cfg):
+        t2 = m.mul(t0, 0.5)
+        t3 = m.add(t2, t1)
+        t4 = m.relu(t3)
+    x0, x1 = make(oracle, (4000, 256), dtype, 31), make(oracle, (4000, 256), dtype, 32)
+    (got,), ex, plan = run_model(m, {t0: x0, t1: x1}, [t4], iters=3)
+    pj = json.loads(plan)
+    assert len(pj["TaskInfos"]) == 1 and len(pj["TaskInfos"][0]["Ops"]) == 3
+    assert pj["TaskInfos"][0]["NumWarps"] == 2
+    ref = oracle.unary(oracle.binary(oracle.scalar(x0, 0.5, "mul", dtype), x1, "add", dtype), "relu", dtype)
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("warps", [1, 2, 4])
+def test_rmsnorm_with_staged_weights_in_narrow_slots(oracle, warps):
+    """RMSNorm stages its fp32 weights in the slot's LDS window and syncs the slot around the copy:
+    with 8 / warps slots per workgroup each slot has a window and a barrier of its own."""
+    from ark_amd import Model
+    dtype, rows, cols = "bf16", 1000, 2048
+    m = Model()
+    x, w = m.tensor((rows, cols), dtype), m.tensor((1, cols), "fp32")
+    cfg = {"NumWarps": warps, "SramBytes": cols * 4, "RowsPerWave": 2, "NumTasks": -(-rows // (warps * 2))}
+    with m.planner_context(config=cfg):
+        y = m.rmsnorm(x, w, eps=1e-6)
+    xs = make(oracle, (rows, cols), dtype, 41)
+    ws = make(oracle, (1, cols), "fp32", 42, "uniform", 0.5, 1.5)
+    (got,), ex, plan = run_model(m, {x: xs, w: ws}, [y], iters=2)
+    assert json.loads(plan)["TaskInfos"][0]["NumWarps"] == warps
+    close(oracle, oracle.rmsnorm(xs, ws.reshape(-1), dtype, eps=1e-6), got, dtype, 1e-2)
