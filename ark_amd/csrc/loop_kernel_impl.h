@@ -168,15 +168,6 @@ __device__ __forceinline__ D load_const(const D *p) {
 
 // FAM is the set of op families compiled into this kernel variant.  A plan runs on the
 // smallest variant that holds its families.
-//
-// The long-running bodies (matmul tiles, skinny matmul, attention) are functions of their own,
-// not inlined into the kernel: each gets its own register allocation and instruction schedule,
-// the same in every variant, in the loop kernel and in the one-op kernels alike.  (Inlined, the
-// K loop of a matmul tile came out differently depending on what surrounded it: in the loop
-// kernel its loads were issued later and it carried five more waits than in a kernel of its
-// own, and ran 10-15 % slower.)  Arguments of a device function arrive in vector registers, so
-// a body takes only indices and reads everything uniform itself: its descriptor from the op
-// table (through the kernel arguments), into scalar registers.
 
 // The small bodies (elementwise ops, row ops, the embedding gather) for one task, inlined.
 template <int FAM>
@@ -220,11 +211,14 @@ __device__ __forceinline__ void run_follower(const DevOp *op, int task, const Sl
 
 // The kernel's one parameter, read where a field is needed: the pointer to the kernel-argument
 // segment is made opaque on every access, so no load from it is shared with an earlier one or
-// lifted out of a loop, and no field occupies a scalar register across an op body (a matmul
-// body needs nearly all of them; with the loop's own state resident beside it the K loop came
-// out with later loads and more waits than the same body in a kernel of its own).
-__device__ __forceinline__ const ARKMI_CONST LoopArgs *kargs() {
-    const ARKMI_CONST LoopArgs *p = (const ARKMI_CONST LoopArgs *)__builtin_amdgcn_kernarg_segment_ptr();
+// lifted out of a loop, and no field occupies a scalar register across an op body.  The pointer
+// is handed down as `ka`: the kernel takes it from the hardware, a non-inlined function gets it
+// as an argument (inside a function the intrinsic yields a null pointer).
+using KArgs = const ARKMI_CONST LoopArgs *;
+
+__device__ __forceinline__ KArgs kernel_kargs() { return (KArgs)__builtin_amdgcn_kernarg_segment_ptr(); }
+
+__device__ __forceinline__ KArgs launder(KArgs p) {
     asm volatile("" : "+s"(p));
     return p;
 }
@@ -240,119 +234,7 @@ __device__ __forceinline__ D load_karg(const ARKMI_CONST D *p) {
     __builtin_memcpy(&d, w, sizeof(D));
     return d;
 }
-#define KARG(field) load_karg(&kargs()->field)
-
-// ---- the long-running bodies -----------------------------------------------------------------
-#ifndef ARKMI_BODY
-#define ARKMI_BODY __device__ __attribute__((noinline))
-#endif
-
-// What a body receives: the address of its op descriptor, the task, the thread index and the
-// address of the workgroup's LDS window (a long-running op owns the whole workgroup, checked on
-// the host).  All but the thread index are uniform and are moved to scalar registers here.  A
-// body must not use the kernel-argument segment: its address is not passed on to a function.
-__device__ __forceinline__ const DevOp *uniform_op(const DevOp *op) {
-    const uint64_t a = reinterpret_cast<uint64_t>(op);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
-    return reinterpret_cast<const DevOp *>(((uint64_t)hi << 32) | lo);
-}
-
-__device__ __forceinline__ Slot body_slot(int tid, lds_ptr lds) {
-    Slot s;
-    s.tid = tid;
-    s.nthreads = kLoopMaxThreads;  // (not read by these bodies)
-    s.lds = (lds_ptr)(uintptr_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
-    s.lds_bytes = 0;
-    s.whole_block = true;
-    return s;
-}
-
-// One matmul tile shape.  Returns the task index the ops fused behind the matmul run for (the
-// tile this workgroup finished), -1 when another workgroup finishes the tile (a split of K).
-template <typename T, int BM, int BN, bool TRANS_B, bool TRANS_A = false, bool DUAL_B = false, bool SPLIT = false>
-ARKMI_BODY int gemm_body(const DevOp *op, int task, int tid, lds_ptr lds) {
-    const GemmDesc g = load_const(&uniform_op(op)->gemm);
-    return gemm_tile<T, BM, BN, TRANS_B, EpilogueStore, TRANS_A, DUAL_B, SPLIT>(
-        g, __builtin_amdgcn_readfirstlane(task), body_slot(tid, lds), EpilogueStore());
-}
-
-ARKMI_BODY int gemm_f32_body(const DevOp *op, int task, int tid, lds_ptr lds) {
-    const GemmDesc g = load_const(&uniform_op(op)->gemm);
-    gemm_f32_dispatch(g, __builtin_amdgcn_readfirstlane(task), body_slot(tid, lds));
-    return task;
-}
-
-ARKMI_BODY int gemv_body(const DevOp *op, int task, int tid, lds_ptr lds) {
-    const GemvDesc d = load_const(&uniform_op(op)->gemv);
-    gemv_dispatch(d, __builtin_amdgcn_readfirstlane(task), body_slot(tid, lds));
-    return task;
-}
-
-ARKMI_BODY int attn_body(const DevOp *op, int task, int tid, lds_ptr lds) {
-    const AttnDesc d = load_const(&uniform_op(op)->attn);
-    attn_dispatch(d, __builtin_amdgcn_readfirstlane(task), body_slot(tid, lds));
-    return task;
-}
-
-template <int FAM, typename T, bool TRANS_B>
-__device__ __forceinline__ int gemm_by_tile(const DevOp *op, int task, int tid, lds_ptr lds) {
-    const int tm = load_const(&op->gemm_tile_m), tn = load_const(&op->gemm_tile_n);
-    if (load_const(&op->gemm.split_k) == 2) {  // 256x256 tiles only (checked on the host)
-        if constexpr ((FAM & FAM_SPLITK) != 0)
-            return gemm_body<T, 256, 256, TRANS_B, false, false, true>(op, task, tid, lds);
-        else
-            return -1;
-    }
-    if constexpr (TRANS_B) {
-        if (load_const(&op->gemm.b2) != nullptr) {  // gate/up pair: 256-wide tiles only (checked on the host)
-            if (tm == 256) return gemm_body<T, 256, 256, true, false, true>(op, task, tid, lds);
-            return gemm_body<T, 128, 256, true, false, true>(op, task, tid, lds);
-        }
-    }
-    if (tm == 256 && tn == 256) return gemm_body<T, 256, 256, TRANS_B>(op, task, tid, lds);
-    if (tm == 128 && tn == 256) return gemm_body<T, 128, 256, TRANS_B>(op, task, tid, lds);
-    if (tm == 256 && tn == 128) return gemm_body<T, 256, 128, TRANS_B>(op, task, tid, lds);
-    return gemm_body<T, 128, 128, TRANS_B>(op, task, tid, lds);
-}
-
-// The first op of a task, of the long-running kind KIND, for one task.  Returns (uniformly) the
-// task index for the ops that follow in the same fused task: `task` itself, except behind a
-// matmul that splits K, where it is the tile this workgroup finished or -1 (none).
-template <int FAM, int KIND>
-__device__ __forceinline__ int run_long(const DevOp *op, int task, int tid, lds_ptr lds) {
-    int follow = task;
-    if constexpr (KIND == DEV_GEMM) {
-        const int dtype = load_const(&op->gemm.dtype);
-        const bool trans_a = load_const(&op->gemm.trans_a) != 0, trans_b = load_const(&op->gemm.trans_b) != 0;
-        if (dtype == 0 || trans_a) {
-            if constexpr ((FAM & FAM_EXT) != 0) {
-                if (dtype == 0) gemm_f32_body(op, task, tid, lds);
-                else if (dtype == 1) {
-                    if (trans_b) gemm_body<f16, 128, 128, true, true>(op, task, tid, lds);
-                    else gemm_body<f16, 128, 128, false, true>(op, task, tid, lds);
-                } else {
-                    if (trans_b) gemm_body<bf16, 128, 128, true, true>(op, task, tid, lds);
-                    else gemm_body<bf16, 128, 128, false, true>(op, task, tid, lds);
-                }
-            }
-        } else if constexpr ((FAM & FAM_GEMM) != 0) {
-            if (dtype == 1) {
-                follow = trans_b ? gemm_by_tile<FAM, f16, true>(op, task, tid, lds)
-                                 : gemm_by_tile<FAM, f16, false>(op, task, tid, lds);
-            } else {
-                follow = trans_b ? gemm_by_tile<FAM, bf16, true>(op, task, tid, lds)
-                                 : gemm_by_tile<FAM, bf16, false>(op, task, tid, lds);
-            }
-            follow = __builtin_amdgcn_readfirstlane(follow);
-        }
-    } else if constexpr (KIND == DEV_GEMV) {
-        if constexpr ((FAM & FAM_GEMV) != 0) gemv_body(op, task, tid, lds);
-    } else if constexpr (KIND == DEV_ATTN) {
-        if constexpr ((FAM & FAM_ATTN) != 0) attn_body(op, task, tid, lds);
-    }
-    return follow;
-}
+#define KARG(field) load_karg(&launder(ka)->field)  // needs a `KArgs ka` in scope
 
 // The tasks of one task_seq<> of the reference (kernel_template.in:11-27: task ids dealt to
 // processors and slots by the formula): the group's parameters and this workgroup's share.
@@ -384,13 +266,20 @@ __device__ __forceinline__ int64_t task_id(const TaskDeal &d, unsigned t) {
     return d.base + (int64_t)d.g.task_s * r + d.round * q;
 }
 
+__device__ __forceinline__ int task_index(const DevTaskGroup &g, int64_t id) {
+    return ((int)id - g.task_b) / g.task_s;
+}
+
 // Before task index `ti` of a consumer group: wait until the producers' row blocks it reads
 // are complete in this iteration.  The data is then read through this XCD's L2 without
 // invalidating it: the host admits the wait in place of a barrier only where no workgroup can
 // have fetched these lines since the last barrier (rows own whole cache lines, and every reader
-// in between waits like this one).  False (uniformly) once `abort` is raised.
-__device__ __forceinline__ bool wait_for_rows(const DevTaskGroup &g, int ti, const Slot &s, unsigned epoch) {
-    volatile int *fail = reinterpret_cast<volatile int *>(g_loop_lds) + 1;
+// in between waits like this one).  False (uniformly) once `abort` is raised.  Whole-workgroup
+// slots only (checked on the host).
+__device__ __forceinline__ bool wait_for_rows(KArgs ka, const DevTaskGroup &g, int ti, int tid, int nthreads,
+                                              unsigned epoch, lds_ptr control) {
+    // (`control`: the start of the workgroup's LDS; a body function gets it from its slot window)
+    volatile __attribute__((address_space(3))) int *fail = (volatile __attribute__((address_space(3))) int *)control + 1;
     const DevWait *waits = KARG(prog.waits) + g.wait_begin;
     const int32_t *spans = KARG(prog.wait_spans) + g.span_begin + 2 * (ti * g.n_waits);
     unsigned *counters = KARG(prog.dep_counters);
@@ -401,7 +290,7 @@ __device__ __forceinline__ bool wait_for_rows(const DevTaskGroup &g, int ti, con
         const DevWait dw = load_const(waits + w);
         const int lo = load_const(spans + 2 * w), hi = load_const(spans + 2 * w + 1);
         const unsigned target = (unsigned)dw.expect * epoch;
-        for (int c = lo + s.tid; c <= hi; c += s.nthreads)
+        for (int c = lo + tid; c <= hi; c += nthreads)
             ok = poll_reached(counters + (size_t)(dw.counter_base + c) * kDepStride, target, ctl, limit) && ok;
     }
     if (!ok) *fail = 1;
@@ -411,7 +300,7 @@ __device__ __forceinline__ bool wait_for_rows(const DevTaskGroup &g, int ti, con
 
 // After task index `ti` of a producer group: every wave's stores have been acknowledged by the
 // L2, the L2 is written back (the release), then the row block's counter grows by one.
-__device__ __forceinline__ void signal_rows(const DevTaskGroup &g, int ti) {
+__device__ __forceinline__ void signal_rows(KArgs ka, const DevTaskGroup &g, int ti) {
     drain_stores_then_barrier();
     if (threadIdx.x == 0) {
         const int block = load_const(KARG(prog.signal_map) + g.signal_begin + ti);
@@ -420,25 +309,184 @@ __device__ __forceinline__ void signal_rows(const DevTaskGroup &g, int ti) {
     }
 }
 
-__device__ __forceinline__ int task_index(const DevTaskGroup &g, int64_t id) {
-    return ((int)id - g.task_b) / g.task_s;
+// ---- the long-running bodies -----------------------------------------------------------------
+// Matmul tiles, the skinny matmul and attention are functions of their own, not inlined into
+// the kernel: each gets its own register allocation and instruction schedule, the same in every
+// variant, in the loop kernel and in the one-op kernels alike.  (Inlined, the K loop of a
+// matmul tile came out differently depending on what surrounded it: in the loop kernel its
+// loads were issued later and it carried five more waits than in a kernel of its own, and ran
+// 10-15 % slower.)  A function that needs most of the vector registers saves and restores the
+// callee-saved half of them around its body (~6 us for a 256x256 tile), so the task loop runs
+// inside the function: it returns when the group's tasks are done, or after one task when ops
+// are fused behind the matmul (those run in the kernel).  Arguments arrive in vector registers;
+// what is uniform is moved to scalar registers first.
+#ifndef ARKMI_BODY
+#define ARKMI_BODY __device__ __attribute__((noinline))
+#endif
+
+constexpr int kTasksDone = -2;     // returned by a body: the group has no more tasks for this workgroup
+constexpr int kTasksAborted = -3;  // a dependency wait gave up
+
+__device__ __forceinline__ KArgs uniform_kargs(KArgs p) {
+    const uint64_t a = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+    return (KArgs)(uintptr_t)(((uint64_t)hi << 32) | lo);
 }
 
-__device__ __forceinline__ void trace_task(const DevTaskGroup &g, int64_t id, int slot_k, int order, const Slot &s) {
+// A long-running op owns the whole workgroup (checked on the host): slot 0, all waves.
+__device__ __forceinline__ Slot body_slot(int tid, lds_ptr lds) {
+    Slot s;
+    s.tid = tid;
+    s.nthreads = kLoopMaxThreads;  // (not read by these bodies)
+    s.lds = (lds_ptr)(uintptr_t)(uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
+    s.lds_bytes = 0;
+    s.whole_block = true;
+    return s;
+}
+
+// The task loop of a group whose first op is long-running, from this workgroup's task number
+// `t0` on.  `one(op, task)` runs the op for one task and returns the task the fused followers
+// run for (-1: none, a split of K that another workgroup finishes).  Nothing of the group's
+// parameters is kept across the op: they are read again for every task.  Returns kTasksDone,
+// kTasksAborted, or -- for a group with followers, after one task -- that task's follow value.
+template <typename One>
+__device__ __forceinline__ int long_task_loop(KArgs ka, int gi, int t0, int tid, unsigned epoch, lds_ptr control,
+                                              One one) {
+    for (unsigned t = (unsigned)t0;; ++t) {
+        int follow;
+        {
+            const TaskDeal d = deal_of(KARG(prog.groups), gi);
+            const DevTaskGroup &g = d.g;
+            const int64_t id = task_id(d, t);
+            if (id >= g.task_e) return kTasksDone;
 #ifndef ARKMI_NO_TRACE
-    TraceRecord *trace = KARG(prog.trace);
-    if (trace && g.trace_offset >= 0 && s.tid == 0) {
-        TraceRecord rec{(int)blockIdx.x, slot_k, order};
-        trace[g.trace_offset + task_index(g, id)] = rec;
-    }
+            TraceRecord *trace = KARG(prog.trace);
+            if (trace && g.trace_offset >= 0 && tid == 0) {
+                TraceRecord rec{(int)blockIdx.x, 0, (int)t};
+                trace[g.trace_offset + task_index(g, id)] = rec;
+            }
 #endif
+            if (KARG(prog.dep_counters) != nullptr && g.n_waits > 0 &&
+                !wait_for_rows(ka, g, task_index(g, id), tid, kLoopMaxThreads, epoch, control))
+                return kTasksAborted;
+            follow = one(KARG(prog.ops) + g.op_begin, (int)id);
+        }
+        const DevTaskGroup g = load_const(KARG(prog.groups) + gi);
+        if (g.op_count > 1) return follow;  // the kernel runs the followers, signals, and calls again
+        // (a matmul that splits K signals for the tile this workgroup finished, if any)
+        if (KARG(prog.dep_counters) != nullptr && g.signal_begin >= 0 && follow >= 0)
+            signal_rows(ka, g, task_index(g, follow));
+    }
+}
+
+template <typename T, int BM, int BN, bool TRANS_B, bool TRANS_A = false, bool DUAL_B = false, bool SPLIT = false>
+ARKMI_BODY int gemm_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, unsigned epoch) {
+    const KArgs ka = uniform_kargs(ka_in);
+    const Slot s = body_slot(tid, lds);
+    return long_task_loop(ka, __builtin_amdgcn_readfirstlane(gi), __builtin_amdgcn_readfirstlane(t0), tid,
+                          __builtin_amdgcn_readfirstlane(epoch), s.lds - kLdsReserved, [&](const DevOp *op, int task) {
+                              const GemmDesc g = load_const(&op->gemm);
+                              return gemm_tile<T, BM, BN, TRANS_B, EpilogueStore, TRANS_A, DUAL_B, SPLIT>(
+                                  g, task, s, EpilogueStore());
+                          });
+}
+
+ARKMI_BODY int gemm_f32_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, unsigned epoch) {
+    const KArgs ka = uniform_kargs(ka_in);
+    const Slot s = body_slot(tid, lds);
+    return long_task_loop(ka, __builtin_amdgcn_readfirstlane(gi), __builtin_amdgcn_readfirstlane(t0), tid,
+                          __builtin_amdgcn_readfirstlane(epoch), s.lds - kLdsReserved, [&](const DevOp *op, int task) {
+                              const GemmDesc g = load_const(&op->gemm);
+                              gemm_f32_dispatch(g, task, s);
+                              return task;
+                          });
+}
+
+ARKMI_BODY int gemv_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, unsigned epoch) {
+    const KArgs ka = uniform_kargs(ka_in);
+    const Slot s = body_slot(tid, lds);
+    return long_task_loop(ka, __builtin_amdgcn_readfirstlane(gi), __builtin_amdgcn_readfirstlane(t0), tid,
+                          __builtin_amdgcn_readfirstlane(epoch), s.lds - kLdsReserved, [&](const DevOp *op, int task) {
+                              const GemvDesc d = load_const(&op->gemv);
+                              gemv_dispatch(d, task, s);
+                              return task;
+                          });
+}
+
+ARKMI_BODY int attn_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, unsigned epoch) {
+    const KArgs ka = uniform_kargs(ka_in);
+    const Slot s = body_slot(tid, lds);
+    return long_task_loop(ka, __builtin_amdgcn_readfirstlane(gi), __builtin_amdgcn_readfirstlane(t0), tid,
+                          __builtin_amdgcn_readfirstlane(epoch), s.lds - kLdsReserved, [&](const DevOp *op, int task) {
+                              const AttnDesc d = load_const(&op->attn);
+                              attn_dispatch(d, task, s);
+                              return task;
+                          });
+}
+
+#define ARKMI_BODY_ARGS ka, gi, t0, tid, lds, epoch
+
+template <int FAM, typename T, bool TRANS_B>
+__device__ __forceinline__ int gemm_by_tile(const DevOp *op, KArgs ka, int gi, int t0, int tid, lds_ptr lds,
+                                            unsigned epoch) {
+    const int tm = load_const(&op->gemm_tile_m), tn = load_const(&op->gemm_tile_n);
+    if (load_const(&op->gemm.split_k) == 2) {  // 256x256 tiles only (checked on the host)
+        if constexpr ((FAM & FAM_SPLITK) != 0)
+            return gemm_body<T, 256, 256, TRANS_B, false, false, true>(ARKMI_BODY_ARGS);
+        else
+            return kTasksDone;
+    }
+    if constexpr (TRANS_B) {
+        if (load_const(&op->gemm.b2) != nullptr) {  // gate/up pair: 256-wide tiles only (checked on the host)
+            if (tm == 256) return gemm_body<T, 256, 256, true, false, true>(ARKMI_BODY_ARGS);
+            return gemm_body<T, 128, 256, true, false, true>(ARKMI_BODY_ARGS);
+        }
+    }
+    if (tm == 256 && tn == 256) return gemm_body<T, 256, 256, TRANS_B>(ARKMI_BODY_ARGS);
+    if (tm == 128 && tn == 256) return gemm_body<T, 128, 256, TRANS_B>(ARKMI_BODY_ARGS);
+    if (tm == 256 && tn == 128) return gemm_body<T, 256, 128, TRANS_B>(ARKMI_BODY_ARGS);
+    return gemm_body<T, 128, 128, TRANS_B>(ARKMI_BODY_ARGS);
+}
+
+// Hands the group's tasks from number t0 on to the body of its first op (of the long-running
+// kind KIND).  Returns (uniformly) what the body returned.
+template <int FAM, int KIND>
+__device__ __forceinline__ int run_long(const DevOp *op, KArgs ka, int gi, int t0, int tid, lds_ptr lds,
+                                        unsigned epoch) {
+    int r = kTasksDone;
+    if constexpr (KIND == DEV_GEMM) {
+        const int dtype = load_const(&op->gemm.dtype);
+        const bool trans_a = load_const(&op->gemm.trans_a) != 0, trans_b = load_const(&op->gemm.trans_b) != 0;
+        if (dtype == 0 || trans_a) {
+            if constexpr ((FAM & FAM_EXT) != 0) {
+                if (dtype == 0) r = gemm_f32_body(ARKMI_BODY_ARGS);
+                else if (dtype == 1)
+                    r = trans_b ? gemm_body<f16, 128, 128, true, true>(ARKMI_BODY_ARGS)
+                                : gemm_body<f16, 128, 128, false, true>(ARKMI_BODY_ARGS);
+                else
+                    r = trans_b ? gemm_body<bf16, 128, 128, true, true>(ARKMI_BODY_ARGS)
+                                : gemm_body<bf16, 128, 128, false, true>(ARKMI_BODY_ARGS);
+            }
+        } else if constexpr ((FAM & FAM_GEMM) != 0) {
+            if (dtype == 1)
+                r = trans_b ? gemm_by_tile<FAM, f16, true>(op, ARKMI_BODY_ARGS) : gemm_by_tile<FAM, f16, false>(op, ARKMI_BODY_ARGS);
+            else
+                r = trans_b ? gemm_by_tile<FAM, bf16, true>(op, ARKMI_BODY_ARGS) : gemm_by_tile<FAM, bf16, false>(op, ARKMI_BODY_ARGS);
+        }
+    } else if constexpr (KIND == DEV_GEMV) {
+        if constexpr ((FAM & FAM_GEMV) != 0) r = gemv_body(ARKMI_BODY_ARGS);
+    } else if constexpr (KIND == DEV_ATTN) {
+        if constexpr ((FAM & FAM_ATTN) != 0) r = attn_body(ARKMI_BODY_ARGS);
+    }
+    return __builtin_amdgcn_readfirstlane(r);
 }
 
 // The task loop of a group of small ops: the program's and the group's parameters stay in
 // registers (`P` was read once for the step).
 template <int FAM>
-__device__ __forceinline__ bool run_small_tasks(const LoopProgram &P, const TaskDeal &d, const Slot &s, int slot_k,
-                                                unsigned epoch) {
+__device__ __forceinline__ bool run_small_tasks(KArgs ka, const LoopProgram &P, const TaskDeal &d, const Slot &s,
+                                                int slot_k, unsigned epoch) {
     const DevTaskGroup &g = d.g;
     const DevOp *ops = P.ops + g.op_begin;
     const bool deps = P.dep_counters != nullptr;
@@ -454,37 +502,29 @@ __device__ __forceinline__ bool run_small_tasks(const LoopProgram &P, const Task
             P.trace[g.trace_offset + task_index(g, id)] = rec;
         }
 #endif
-        if (waits && !wait_for_rows(g, ti, s, epoch)) return false;
+        if (waits && !wait_for_rows(ka, g, ti, s.tid, s.nthreads, epoch, (lds_ptr)g_loop_lds)) return false;
         for (int o = 0; o < g.op_count; ++o) {
             // later ops of a fused task read what earlier ones of the same slot wrote: the slot's
             // waves meet (they share one L1, which sees their stores)
             if (o > 0) s.sync();
             run_small<FAM>(ops + o, (int)id, s);
         }
-        if (signals) signal_rows(g, ti);
+        if (signals) signal_rows(ka, g, ti);
     }
     return true;
 }
 
-// The task loop of a group whose first op is long-running (KIND: matmul, skinny matmul,
-// attention), one loop per kind, so what the compiler lifts out of a loop stays live across
-// that body only.  Nothing of the group's parameters is kept across the body: they are read
-// again for every task.
+// A group whose first op is long-running (KIND: matmul, skinny matmul, attention): the body
+// function runs the tasks; it comes back after each task when ops are fused behind a matmul,
+// which then run here.
 template <int FAM, int KIND>
-__device__ __forceinline__ bool run_long_tasks(int gi, const Slot &s, int slot_k, unsigned epoch) {
-    int order = 0;
-    for (unsigned t = (unsigned)slot_k;; ++order) {
-        int follow;
-        {
-            const TaskDeal d = deal_of(KARG(prog.groups), gi);
-            const DevTaskGroup &g = d.g;
-            const int64_t id = task_id(d, t);
-            if (id >= g.task_e) break;
-            const bool deps = KARG(prog.dep_counters) != nullptr;
-            trace_task(g, id, slot_k, order, s);
-            if (deps && g.n_waits > 0 && !wait_for_rows(g, task_index(g, id), s, epoch)) return false;
-            follow = run_long<FAM, KIND>(KARG(prog.ops) + g.op_begin, (int)id, s.tid, s.lds);  // uniform across the workgroup
-        }
+__device__ __forceinline__ bool run_long_tasks(KArgs ka, int gi, const Slot &s, unsigned epoch) {
+    for (int t = 0;; ++t) {
+        const DevOp *first = KARG(prog.ops) + load_const(&(KARG(prog.groups) + gi)->op_begin);
+        const int follow = run_long<FAM, KIND>(first, ka, gi, t, s.tid, s.lds, epoch);
+        if (follow == kTasksDone) return true;
+        if (follow == kTasksAborted) return false;
+        // one task of a group with followers was run; `follow` is the tile they run for
         const DevTaskGroup g = load_const(KARG(prog.groups) + gi);
         if constexpr (KIND == DEV_GEMM) {
             const DevOp *ops = KARG(prog.ops) + g.op_begin;
@@ -493,12 +533,9 @@ __device__ __forceinline__ bool run_long_tasks(int gi, const Slot &s, int slot_k
                 run_follower<FAM>(ops + o, follow, s);
             }
         }
-        // (a matmul that splits K signals for the tile this workgroup finished, if any)
         if (KARG(prog.dep_counters) != nullptr && g.signal_begin >= 0 && follow >= 0)
-            signal_rows(g, task_index(g, follow));
-        t += (unsigned)g.n_slots;
+            signal_rows(ka, g, task_index(g, follow));
     }
-    return true;
 }
 
 // Does this variant hold a long-running body?  If not, nothing competes for scalar registers
@@ -509,7 +546,7 @@ constexpr bool kHasLongBodies = (FAM & (FAM_GEMM | FAM_SPLITK | FAM_EXT | FAM_GE
 constexpr int kLdsSlotCounters = 64;  // byte offset of the slots' arrival counters in the control area
 
 template <int FAM>
-__device__ __forceinline__ bool run_group(const LoopProgram &P, int gi, unsigned epoch) {
+__device__ __forceinline__ bool run_group(KArgs ka, const LoopProgram &P, int gi, unsigned epoch) {
     const TaskDeal d = deal_of(P.groups, gi);
     const DevTaskGroup &g = d.g;
     if (!d.mine) return true;
@@ -527,17 +564,17 @@ __device__ __forceinline__ bool run_group(const LoopProgram &P, int gi, unsigned
     // (a variant holds the loops of the families it was built for)
     const int first = load_const(&(P.ops + g.op_begin)->kind);
     if constexpr ((FAM & (FAM_GEMM | FAM_SPLITK | FAM_EXT)) != 0) {
-        if (first == DEV_GEMM) return run_long_tasks<FAM, DEV_GEMM>(gi, s, k, epoch);
+        if (first == DEV_GEMM) return run_long_tasks<FAM, DEV_GEMM>(ka, gi, s, epoch);
     }
     if constexpr ((FAM & FAM_GEMV) != 0) {
-        if (first == DEV_GEMV) return run_long_tasks<FAM, DEV_GEMV>(gi, s, k, epoch);
+        if (first == DEV_GEMV) return run_long_tasks<FAM, DEV_GEMV>(ka, gi, s, epoch);
     }
     if constexpr ((FAM & FAM_ATTN) != 0) {
-        if (first == DEV_ATTN) return run_long_tasks<FAM, DEV_ATTN>(gi, s, k, epoch);
+        if (first == DEV_ATTN) return run_long_tasks<FAM, DEV_ATTN>(ka, gi, s, epoch);
     }
     if constexpr ((FAM & (FAM_ROW | FAM_EWISE | FAM_EXT)) != 0) {
         if (first != DEV_GEMM && first != DEV_GEMV && first != DEV_ATTN)
-            return run_small_tasks<FAM>(P, d, s, k, epoch);
+            return run_small_tasks<FAM>(ka, P, d, s, k, epoch);
     }
     return true;
 }
@@ -552,7 +589,7 @@ __device__ __forceinline__ void init_lds_control() {
 
 // One iteration of the plan's body; `epoch` counts the iterations since the launch from 1.
 template <int FAM>
-__device__ __forceinline__ bool run_body(const LoopProgram &P0, XcdInfo &xi, unsigned epoch) {
+__device__ __forceinline__ bool run_body(KArgs ka, const LoopProgram &P0, XcdInfo &xi, unsigned epoch) {
     const int num_steps = kHasLongBodies<FAM> ? KARG(prog.num_steps) : P0.num_steps;
     for (int si = 0; si < num_steps; ++si) {
         // (one read of the whole parameter block per step where long bodies want the registers)
@@ -571,7 +608,7 @@ __device__ __forceinline__ bool run_body(const LoopProgram &P0, XcdInfo &xi, uns
             // L1, which sees their own stores, so the workgroup only has to meet
             __syncthreads();
         } else {
-            if (!run_group<FAM>(P, st.index, epoch)) return false;
+            if (!run_group<FAM>(ka, P, st.index, epoch)) return false;
         }
     }
     unsigned long long *clock = KARG(prog.step_clock);
@@ -581,6 +618,7 @@ __device__ __forceinline__ bool run_body(const LoopProgram &P0, XcdInfo &xi, uns
 
 template <int FAM>
 __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(LoopArgs) {
+    const KArgs ka = kernel_kargs();
     const unsigned nblocks = gridDim.x;
     const bool leader = (blockIdx.x == 0 && threadIdx.x == 0);
     init_lds_control();
@@ -653,7 +691,7 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(LoopArgs) {
                 }
             }
             ++epoch;
-            if (ok) ok = run_body<FAM>(P0, xi, epoch);
+            if (ok) ok = run_body<FAM>(ka, P0, xi, epoch);
         }
         if (!ok) break;
         // results must be visible to the host before the command is cleared: every
@@ -682,9 +720,10 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_loop_kernel(LoopArgs) {
 // boundaries order everything.
 template <int FAM>
 __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_step_kernel(LoopArgs) {
+    const KArgs ka = kernel_kargs();
     init_lds_control();
     const LoopProgram P = KARG(prog);
-    run_group<FAM>(P, KARG(group), 1u);
+    run_group<FAM>(ka, P, KARG(group), 1u);
 }
 
 // Defines the host-visible handles of one kernel variant; each variant is its own
