@@ -555,6 +555,13 @@ __device__ __forceinline__ bool run_group(KArgs ka, const LoopProgram &P, int gi
     if (k >= g.n_slots) return true;
     Slot s;
     s.tid = threadIdx.x - k * slot_threads;
+    // Opaque per task group: what the bodies derive from the thread index alone (per-lane
+    // address parts) is loop-invariant for the compiler, which would lift it out of the step and
+    // iteration loops for every body at once and keep it live across all of them and across the
+    // calls of the long-running bodies, where only the callee-saved registers survive (one
+    // variant spilled 51 000 vector registers that way).  Inside the group's task loop it may
+    // still be lifted.
+    asm volatile("" : "+v"(s.tid));
     s.nthreads = slot_threads;
     s.lds = (lds_ptr)g_loop_lds + kLdsReserved + k * g.slot_sram;
     s.lds_bytes = g.slot_sram;

@@ -1,4 +1,7 @@
 // Loop-kernel variant: elementwise + GEMM incl. the split of K.
+// Bodies inlined: this variant mixes long-running and small bodies, and with the long ones as
+// functions the register allocation of the small ones around the call sites was measured worse.
+#define ARKMI_BODY __device__ __forceinline__
 #include "loop_kernel_impl.h"
 namespace arkmi {
 ARKMI_LOOP_KERNEL_VARIANT(70)

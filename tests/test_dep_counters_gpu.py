@@ -1,6 +1,6 @@
 """Dependency counters in place of grid barriers (the loop kernel's per-row-block counters in
 device memory): each graph runs with the counters and with every barrier kept
-(ARKMI_DEP_COUNTERS=0); outputs must agree bit for bit over several iterations, in the resident
+(ARKMI_DEP_COUNTERS=0, the default); outputs must agree bit for bit over several iterations, in the resident
 loop kernel and in one-shot launches, and the executor must report which barriers it replaced.
 The reference orders the same chains with one sync_gpu per op boundary (ark/codegen.cpp:109-158)."""
 import numpy as np
@@ -116,3 +116,31 @@ def test_counters_across_commands_and_relaunch(oracle, monkeypatch):
             ex.wait()
             assert np.array_equal(ex.tensor_read(fetch[0]), want), (launch, n)
         ex.stop()
+
+
+@pytest.mark.parametrize("fused", [True, "attention"])
+def test_decoder_layer_with_counters(oracle, fused, monkeypatch):
+    """The fused Llama decoder layer (RMSNorm -> projections with the rotation on their tiles ->
+    attention -> output projection with the residual -> RMSNorm -> SwiGLU -> down projection with the
+    residual): with counters every barrier of the chain is replaced; results bit for bit."""
+    import test_llama_gpu as L
+    from ark_amd import Model
+    dtype, seq, dim, heads, hidden = "bf16", 2048, 4096, 32, 11008  # the size at which every op fills the grid
+    results = {}
+    for counters in ("0", "1"):
+        monkeypatch.setenv("ARKMI_DEP_COUNTERS", counters)
+        m = Model()
+        blk, vals, x, freqs, mask = L._layer_case(oracle, m, seq, dim, heads, hidden, dtype, 600)
+        tx = m.tensor([1, seq, dim], dtype)
+        tf = m.tensor([1, seq, 1, dim // heads], dtype)
+        tm = m.tensor([1, 1, seq, seq], dtype)
+        out = blk.forward(tx, tf, tm, fused=bool(fused), causal=(fused == "attention"))
+        feeds = {tx: x, tf: oracle.to_storage(freqs, dtype), tm: oracle.to_storage(mask, dtype)}
+        if fused == "attention":
+            del feeds[tm]
+        feeds.update({t: vals[name] for name, t in blk.params().items()})
+        (got,), info = _run(m, feeds, [out], iters=2)
+        if counters == "1":
+            assert info["barriers_counted"] >= 4, info
+        results[counters] = got
+    assert np.array_equal(results["0"], results["1"])
