@@ -1,5 +1,8 @@
 // Loop-kernel variant: the rarely used bodies (fp32 / transposed-first-operand matmul, reductions over
 // an axis other than the last), also as a one-op kernel.
+// Bodies inlined: a function that needs most vector registers saves and restores over a hundred
+// of them per call (~8 us), too much beside a body that runs for 20-100 us.
+#define ARKMI_BODY __device__ __forceinline__
 #include "loop_kernel_impl.h"
 namespace arkmi {
 ARKMI_LOOP_KERNEL_VARIANT(32)
