@@ -271,6 +271,15 @@ def config_c5(torch, np, Model, Executor, llama, inp, cpu):
         plan = m.plan(device_id=0)
         loop_us, info = _resident_us(torch, Executor, plan, 10, feeds)
         one_us, sep_us = _oneshot_and_separate_us(torch, Executor, plan, 10, feeds)
+        counters = None
+        if fused == "attention":
+            # the same plan with its grid barriers replaced by dependency counters (off by default)
+            os.environ["ARKMI_DEP_COUNTERS"] = "1"
+            try:
+                dep_us, dep_info = _resident_us(torch, Executor, plan, 10, feeds)
+            finally:
+                del os.environ["ARKMI_DEP_COUNTERS"]
+            counters = {"resident_loop_kernel_us": round(dep_us, 1), "barriers_counted": dep_info["barriers_counted"]}
         # full (unskipped) attention counts 897.7 GFLOP; the attention op skips the masked key blocks
         fl = 863.3e9 if fused == "attention" else 897.7e9
         base = None
@@ -295,6 +304,8 @@ def config_c5(torch, np, Model, Executor, llama, inp, cpu):
             + {False: "the reference's op-by-op composition", True: "fused ops, matmul/softmax attention",
                "attention": "fused ops, attention as one op; flop count with masked key blocks skipped"}[fused] + ")",
             "mfma", fl, one_us, loop_us, sep_us, info, base)
+        if counters:
+            out[names[fused]]["with_dependency_counters"] = counters
     return out
 
 
