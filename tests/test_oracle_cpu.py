@@ -305,3 +305,24 @@ def test_plan_oracle_task_ids_agree_with_c(oracle):
     for block in range(8):
         for k in range(2):
             assert P.task_ids(step, block, 8, k) == oracle.task_seq(block, 8, (0, 6, 1), 2, (0, 50, 1), 2, 2, k)
+
+
+def test_embedding_oracle_by_brute_force(oracle):
+    """The gather restated from ark/ops/ops_embedding_test.cpp:11-41, checked element by element
+    with plain loops on a tiny case, negative indices (counted from the end of the table) included,
+    and against the one-hot matrix product that defines an embedding lookup."""
+    rng = np.random.default_rng(3)
+    table = rng.standard_normal((7, 5)).astype(np.float32)
+    idx = np.array([[0, 6, -1], [3, -7, 2]], dtype=np.int32)
+    got = oracle.embedding(idx, table)
+    assert got.shape == (2, 3, 5)
+    for i in range(2):
+        for j in range(3):
+            row = int(idx[i, j])
+            row = row + 7 if row < 0 else row
+            for c in range(5):
+                assert got[i, j, c] == table[row, c]
+    onehot = np.zeros((6, 7), np.float32)
+    flat = np.where(idx.reshape(-1) < 0, idx.reshape(-1) + 7, idx.reshape(-1))
+    onehot[np.arange(6), flat] = 1.0
+    assert np.array_equal(got.reshape(6, 5), onehot @ table)
