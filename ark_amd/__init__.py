@@ -7,7 +7,7 @@ side over that ABI; PyTorch is used only for device memory and streams.
 from ._lib import lib, check, ArkmiError, DTYPES, device_info  # noqa: F401
 from . import ops  # noqa: F401
 from .model import Model, Tensor, PlannerContext, reset_ids  # noqa: F401
-from .executor import Executor, plan_schedule, schedule_tasks  # noqa: F401
+from .executor import Executor, plan_schedule, plan_analysis, schedule_tasks  # noqa: F401
 
 
 def init():

@@ -1090,6 +1090,14 @@ struct Executor {
     int barriers_elided = 0;
     int barriers_local = 0;       // grid barriers replaced by a workgroup-local sync
     int barriers_counted = 0;     // grid barriers replaced by waits on dependency counters
+    // Analysis only (no device): compile() stops before anything touches the GPU and keeps the
+    // tables it built.  force_deps: -1 take ARKMI_DEP_COUNTERS, 0 / 1 override it.
+    bool dry = false;
+    int force_deps = -1;
+    std::vector<DevStep> dry_steps;
+    std::vector<DevWait> dry_waits;
+    std::vector<int32_t> dry_spans, dry_signal;
+    size_t dry_counters = 0;
     DevWait *d_waits = nullptr;
     int32_t *d_spans = nullptr, *d_signal = nullptr;
     unsigned int *d_dep_counters = nullptr;
@@ -1187,7 +1195,7 @@ struct Executor {
     void compile() {
         if (destroyed) ARK_ERR(InvalidUsageError, "executor is destroyed");
         if (compiled) return;
-        set_device();
+        if (!dry) set_device();
         const int block_warps = sched.num_warps_per_processor;
         threads = block_warps * 64;
         grid = sched.num_processors;
@@ -1196,6 +1204,12 @@ struct Executor {
                     kLoopMaxThreads / 64, " waves per workgroup");
         Lowering L{arena, buffer_offset, [this](size_t bytes) {
                        void *p = nullptr;
+                       if (dry) {  // addresses are only computed with, never followed
+                           static uintptr_t next = (uintptr_t)1 << 46;
+                           p = (void *)next;
+                           next += (bytes + 255) / 256 * 256;
+                           return p;
+                       }
                        ARKMI_HIP(hipMalloc(&p, bytes));
                        ARKMI_HIP(hipMemset(p, 0, bytes));
                        scratch_allocs.push_back(p);
@@ -1378,7 +1392,7 @@ struct Executor {
             // (each signal is an L2 write-back, the wait for the slowest producer stays, and the
             // iteration boundary needs its barrier back), measured 1169 against 1144 us.
             const char *dep_env = getenv("ARKMI_DEP_COUNTERS");
-            bool use_deps = elide && dep_env && atoi(dep_env) != 0;
+            bool use_deps = elide && (force_deps >= 0 ? force_deps != 0 : (dep_env && atoi(dep_env) != 0));
             for (const auto &st : sched.steps)
                 if (st.is_barrier && !(st.b == 0 && st.e >= grid)) use_deps = false;
             std::vector<DepGroup> dg;
@@ -1448,7 +1462,16 @@ struct Executor {
                         dg[(size_t)yi].waits.clear();
                         std::vector<int> rest;
                         for (int xi : window)
-                            if ((size_t)dg[(size_t)xi].sched_step > keep) rest.push_back(xi);
+                            if ((size_t)dg[(size_t)xi].sched_step > keep) {
+                                rest.push_back(xi);
+                                // the barrier now orders these groups after everything ahead of it
+                                auto &ws = dg[(size_t)xi].waits;
+                                ws.erase(std::remove_if(ws.begin(), ws.end(),
+                                                        [&](const DepGroup::Wait &w) {
+                                                            return (size_t)dg[(size_t)w.producer].sched_step < keep;
+                                                        }),
+                                         ws.end());
+                            }
                         window.swap(rest);
                     }
                     window.push_back(yi);
@@ -1557,6 +1580,15 @@ struct Executor {
         // invalidated since the previous one
         if (barriers_counted > 0) iteration_sync = 2;
         lds_bytes = loop_kernel_lds_reserved() + max_slot_lds;
+        if (dry) {
+            (void)loop_kernel_select(families, &kernel_families);
+            dry_steps = steps;
+            dry_waits = h_waits;
+            dry_spans = h_spans;
+            dry_signal = h_signal;
+            dry_counters = n_counters;
+            return;
+        }
         const auto &facts = device_facts(device);
         if (lds_bytes > facts.lds_bytes)
             ARK_ERR(PlanError, "plan needs ", lds_bytes, " bytes of LDS per workgroup; the CU has ",
@@ -2069,6 +2101,92 @@ int arkmi_exec_read_step_clocks(arkmi_exec *h, uint64_t *ticks, size_t max_entri
         if (!ticks) return;
         auto clk = schedule_clocks(ex);
         std::memcpy(ticks, clk.data(), std::min(max_entries, clk.size()) * sizeof(uint64_t));
+    });
+}
+
+int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis_json) {
+    return guard_exec([&] {
+        if (!plan_json || !analysis_json) ARK_ERR(InvalidUsageError, "null argument");
+        arkmi::Executor ex;
+        ex.dry = true;
+        ex.force_deps = dep_counters;
+        try {
+            ex.plan = Json::parse(plan_json);
+        } catch (const std::exception &e) {
+            ARK_ERR(PlanError, "failed to parse the plan: ", e.what());
+        }
+        ex.plan_text = plan_json;
+        ex.sched = arkmi::build_schedule(ex.plan);
+        ex.layout_buffers();
+        ex.arena = (char *)((uintptr_t)1 << 45);  // a stand-in base address: nothing is read through it
+        try {
+            ex.compile();
+        } catch (...) {
+            ex.arena = nullptr;
+            ex.destroyed = true;
+            throw;
+        }
+        ex.arena = nullptr;
+        ex.destroyed = true;  // nothing to release
+        Json out = Json::object();
+        out["NumProcessors"] = (long long)ex.grid;
+        out["KernelFamilies"] = (long long)ex.kernel_families;
+        out["BarriersElided"] = (long long)ex.barriers_elided;
+        out["BarriersLocal"] = (long long)ex.barriers_local;
+        out["BarriersCounted"] = (long long)ex.barriers_counted;
+        out["IterationSync"] = (long long)ex.iteration_sync;
+        out["NumCounters"] = (long long)ex.dry_counters;
+        Json steps = Json::array();
+        for (const auto &st : ex.dry_steps) {
+            Json j = Json::object();
+            if (st.kind == arkmi::STEP_BARRIER) {
+                j["Kind"] = "Barrier";
+                j["Count"] = (long long)st.count;
+            } else if (st.kind == arkmi::STEP_LOCAL_SYNC) {
+                j["Kind"] = "LocalSync";
+            } else {
+                const arkmi::DevTaskGroup &g = ex.h_groups[(size_t)st.index];
+                const int n_tasks = std::max(0, (g.task_e - g.task_b + g.task_s - 1) / g.task_s);
+                j["Kind"] = "Tasks";
+                j["Group"] = (long long)st.index;
+                j["NumTasks"] = (long long)n_tasks;
+                Json waits = Json::array();
+                for (int w = 0; w < g.n_waits; ++w) {
+                    const arkmi::DevWait &dw = ex.dry_waits[(size_t)(g.wait_begin + w)];
+                    Json jw = Json::object();
+                    long long producer = -1;
+                    for (size_t gi = 0; gi < ex.h_groups.size(); ++gi)
+                        if (ex.h_groups[gi].signal_begin >= 0 && ex.h_groups[gi].signal_base == dw.counter_base)
+                            producer = (long long)gi;
+                    jw["ProducerGroup"] = producer;
+                    jw["Expect"] = (long long)dw.expect;
+                    Json spans = Json::array();
+                    for (int t = 0; t < n_tasks; ++t) {
+                        Json sp = Json::array();
+                        sp.push_back((long long)ex.dry_spans[(size_t)(g.span_begin + 2 * (t * g.n_waits + w))]);
+                        sp.push_back((long long)ex.dry_spans[(size_t)(g.span_begin + 2 * (t * g.n_waits + w) + 1)]);
+                        spans.push_back(sp);
+                    }
+                    jw["Spans"] = spans;
+                    waits.push_back(jw);
+                }
+                j["Waits"] = waits;
+                if (g.signal_begin >= 0 && ex.barriers_counted > 0) {
+                    Json map = Json::array();
+                    int n_signal = n_tasks;
+                    // (a matmul that splits K signals once per tile)
+                    size_t end = ex.dry_signal.size();
+                    for (const auto &g2 : ex.h_groups)
+                        if (g2.signal_begin > g.signal_begin) end = std::min(end, (size_t)g2.signal_begin);
+                    n_signal = (int)(end - (size_t)g.signal_begin);
+                    for (int t = 0; t < n_signal; ++t) map.push_back((long long)ex.dry_signal[(size_t)(g.signal_begin + t)]);
+                    j["SignalMap"] = map;
+                }
+            }
+            steps.push_back(j);
+        }
+        out["Steps"] = steps;
+        *analysis_json = dup_text(out.dump());
     });
 }
 

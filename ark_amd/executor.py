@@ -43,6 +43,17 @@ def plan_schedule(plan):
         lib().arkmi_free(out)
 
 
+def plan_analysis(plan, dep_counters=-1):
+    """What compile() decides for the plan (no GPU needed): barriers kept, elided, made local or
+    replaced by dependency counters, and the counters' wait and signal tables."""
+    out = ctypes.c_char_p()
+    check(lib().arkmi_plan_analysis(plan.encode(), ctypes.c_int(dep_counters), ctypes.byref(out)))
+    try:
+        return json.loads(ctypes.string_at(out).decode())
+    finally:
+        lib().arkmi_free(out)
+
+
 def schedule_tasks(plan, step, block, slot):
     """Task ids (block, slot) runs in schedule step `step` (no GPU needed)."""
     n = ctypes.c_int()

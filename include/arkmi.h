@@ -312,6 +312,14 @@ int arkmi_exec_read_step_clocks(arkmi_exec *h, uint64_t *ticks,
                                 size_t max_entries, int *n_blocks,
                                 int *n_steps, int *ticks_per_ms);
 
+/* What compile() decides for a plan, without a GPU: the device steps (grid barriers kept, workgroup
+ * syncs, task groups), the barrier statistics of arkmi_exec_info_t, and -- with dep_counters 1 (0: off,
+ * -1: as ARKMI_DEP_COUNTERS says) -- the dependency counters: per consumer group the producer group, the
+ * expected count per iteration and the counter span [lo, hi] each task waits for; per producer group
+ * the row block each task signals.  Counterpart of reading the generated kernel source of the reference
+ * (ark/codegen.cpp:109-158 places its sync_gpu calls there).  Free the text with arkmi_free. */
+int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis_json);
+
 /* The schedule a plan compiles to, as JSON: the ordered barriers and
  * task_seq<> argument lists the reference's code generator would emit
  * (ark/codegen.cpp:109-158,272-400).  No GPU needed. */

@@ -1,0 +1,143 @@
+"""The host side of the dependency counters without a GPU (arkmi_plan_analysis): which barriers
+compile() replaces by counters, and the wait spans / signal maps it builds, recomputed here from
+first principles (task -> rows by the ops' own tiling rules) for every task of the plans.
+The reference places one sync_gpu between consecutive ops instead (ark/codegen.cpp:109-158)."""
+import json
+
+import pytest
+
+from ark_amd import Model, llama, plan_analysis
+
+
+def _plan(m):
+    return m.plan(arch="ROCM_950", num_processors=256)
+
+
+def _tasks_steps(a):
+    return [s for s in a["Steps"] if s["Kind"] == "Tasks"]
+
+
+def _cfg(plan, task_info, op=0):
+    return json.loads(plan)["TaskInfos"][task_info]["Ops"][op]["Config"]
+
+
+def test_rows_feeding_matmuls_spans_by_first_principles():
+    m = Model()
+    x, w1, w2 = m.tensor([4096, 2048], "fp16"), m.tensor([2048, 4096], "fp16"), m.tensor([4096, 2048], "fp16")
+    m.matmul(m.matmul(m.rmsnorm(x), w1), w2)
+    plan = _plan(m)
+    off = plan_analysis(plan, 0)
+    assert off["BarriersCounted"] == 0 and off["NumCounters"] == 0
+    assert [s["Kind"] for s in off["Steps"]] == ["Tasks", "Barrier", "Tasks", "Barrier", "Tasks"]
+    a = plan_analysis(plan, 1)
+    assert a["BarriersCounted"] == 2 and a["IterationSync"] == 2
+    assert [s["Kind"] for s in a["Steps"]] == ["Tasks", "LocalSync", "Tasks", "LocalSync", "Tasks"]
+    norm, mm1, mm2 = _tasks_steps(a)
+    # producer 0: RMSNorm, a task covers NumWarps x RowsPerWave rows and signals its own block
+    c0 = _cfg(plan, 0)
+    rows_per_task = c0["NumWarps"] * c0["RowsPerWave"]
+    assert norm["NumTasks"] == 4096 // rows_per_task and norm["SignalMap"] == list(range(norm["NumTasks"]))
+    assert norm["Waits"] == []
+    # consumer 1: tile t reads the rows of its tile row (tile index row-major, N fastest)
+    c1 = _cfg(plan, 1)
+    bm, bn = c1["TileShapeMNK"][:2]
+    tiles_n = 4096 // bn
+    (w,) = mm1["Waits"]
+    assert w["ProducerGroup"] == norm["Group"] and w["Expect"] == 1
+    for t, (lo, hi) in enumerate(w["Spans"]):
+        r0, r1 = (t // tiles_n) * bm, (t // tiles_n + 1) * bm
+        assert (lo, hi) == (r0 // rows_per_task, (r1 - 1) // rows_per_task), t
+    # producer 1 signals the block of its tile row; every block collects one signal per tile column
+    assert mm1["SignalMap"] == [t // tiles_n for t in range(mm1["NumTasks"])]
+    # consumer 2 waits for the tile rows of the first matmul that cover its own rows
+    c2 = _cfg(plan, 2)
+    bm2, bn2 = c2["TileShapeMNK"][:2]
+    tiles_n2 = 2048 // bn2
+    (w,) = mm2["Waits"]
+    assert w["ProducerGroup"] == mm1["Group"] and w["Expect"] == tiles_n
+    for t, (lo, hi) in enumerate(w["Spans"]):
+        r0, r1 = (t // tiles_n2) * bm2, (t // tiles_n2 + 1) * bm2
+        assert (lo, hi) == (r0 // bm, (r1 - 1) // bm), t
+    assert "SignalMap" not in mm2  # nobody waits for the last group
+    assert a["NumCounters"] == norm["NumTasks"] + 4096 // bm
+
+
+def test_write_after_read_keeps_the_last_barrier():
+    """x <- x + 0.01 * (rmsnorm(x) @ w): the final add overwrites what the RMSNorm read, a hazard no
+    counter expresses, so the barrier ahead of the add stays and the groups behind it start a new
+    window; the barriers ahead of it are counted."""
+    m = Model()
+    x, w = m.tensor([16384, 2048], "fp16"), m.tensor([2048, 2048], "fp16")
+    h = m.matmul(m.rmsnorm(x), w)
+    m.add(x, m.mul(h, 0.01), output=x)
+    a = plan_analysis(_plan(m), 1)
+    kinds = [s["Kind"] for s in a["Steps"]]
+    assert kinds.count("Tasks") == 4
+    # RMSNorm -> matmul is counted; the barrier ahead of the scalar multiply stays (it is the last
+    # full barrier between the reader of x and its writer: the multiply and the add share tiles, so
+    # the barrier between those two was a workgroup sync already)
+    assert kinds == ["Tasks", "LocalSync", "Tasks", "Barrier", "Tasks", "LocalSync", "Tasks"]
+    assert a["Steps"][3]["Count"] == 256 and a["BarriersCounted"] == 1
+    norm, mm, mul, add = _tasks_steps(a)
+    assert [w["ProducerGroup"] for w in mm["Waits"]] == [norm["Group"]]
+    assert mul["Waits"] == [] and add["Waits"] == []  # ordered by the barrier, not by counters
+    assert "SignalMap" not in mm
+
+
+def test_sub_grid_barriers_are_never_replaced():
+    m = Model()
+    """RMSNorm on 64 processors, then two matmuls of 16 tiles: the barrier between the matmuls spans
+    16 of the plan's 64 processors.  A plan with such a barrier keeps all of them (the argument for
+    reading without a cache invalidate needs every workgroup at every barrier that stays)."""
+    x, w = m.tensor([512, 512], "fp16"), m.tensor([512, 512], "fp16")
+    m.matmul(m.matmul(m.rmsnorm(x), w), w)
+    a = plan_analysis(_plan(m), 1)
+    assert a["NumProcessors"] == 64
+    assert a["BarriersCounted"] == 0 and a["NumCounters"] == 0
+    assert sorted(s["Count"] for s in a["Steps"] if s["Kind"] == "Barrier") == [16, 64]
+
+
+def test_decoder_layer_replaces_every_barrier():
+    m = Model()
+    blk = llama.TransformerBlock(m, 4096, 32, 11008, "bf16")
+    tx = m.tensor([1, 2048, 4096], "bf16")
+    tf = m.tensor([1, 2048, 1, 128], "bf16")
+    tm = m.tensor([1, 1, 2048, 2048], "bf16")
+    blk.forward(tx, tf, tm, fused=True, causal=True)
+    plan = _plan(m)
+    off, on = plan_analysis(plan, 0), plan_analysis(plan, 1)
+    assert off["BarriersCounted"] == 0 and [s["Kind"] for s in off["Steps"]].count("Barrier") == 6
+    assert on["BarriersCounted"] == 6 and "Barrier" not in [s["Kind"] for s in on["Steps"]]
+    assert on["KernelFamilies"] == off["KernelFamilies"] == 87
+    groups = _tasks_steps(on)
+    names = ["norm1", "q", "k", "v", "attn", "wo", "norm2", "swiglu", "down"]
+    g = dict(zip(names, groups))
+    # the three projections wait for the first RMSNorm only, and not for each other
+    for p in ("q", "k", "v"):
+        assert [w["ProducerGroup"] for w in g[p]["Waits"]] == [g["norm1"]["Group"]]
+    # attention: the query block's rows of Q, and K / V up to the causal diagonal (128-row blocks)
+    waits = {w["ProducerGroup"]: w for w in g["attn"]["Waits"]}
+    assert sorted(waits) == [g["q"]["Group"], g["k"]["Group"], g["v"]["Group"]]
+    qb_count = 2048 // 128
+    for t in range(g["attn"]["NumTasks"]):
+        bh, qb = divmod(t, qb_count)
+        if bh >= 16:  # the upper half of the heads runs its query blocks backwards
+            qb = qb_count - 1 - qb
+        assert tuple(waits[g["q"]["Group"]]["Spans"][t]) == (qb, qb), t
+        assert tuple(waits[g["k"]["Group"]]["Spans"][t]) == (0, qb), t
+        assert tuple(waits[g["v"]["Group"]]["Spans"][t]) == (0, qb), t
+    # every projection block expects one signal per tile column (4096 / 256 = 16 tiles)
+    assert all(w["Expect"] == 16 for w in waits.values())
+    # the output projection reads all heads of its rows: 128 query rows = 32 attention tasks per block
+    (w,) = g["wo"]["Waits"]
+    assert w["ProducerGroup"] == g["attn"]["Group"] and w["Expect"] == 32
+    # the down projection needs the SwiGLU rows of its tile and the residual it adds
+    assert sorted(w["ProducerGroup"] for w in g["down"]["Waits"]) == sorted([g["wo"]["Group"], g["swiglu"]["Group"]])
+    assert "SignalMap" not in g["down"]
+
+
+def test_analysis_rejects_what_compile_rejects():
+    from ark_amd import ArkmiError
+    with pytest.raises(ArkmiError) as e:
+        plan_analysis("{not json", 1)
+    assert e.value.kind == "PlanError"
