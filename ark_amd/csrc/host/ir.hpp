@@ -6,6 +6,7 @@
 // one C++ class per op type, an op here is a plain record (type name, tensors,
 // args); per-type behaviour lives in function tables (host/ops.cpp).
 #pragma once
+#include <ark/log.hpp>
 #include <unistd.h>
 
 #include <ark/dims.hpp>
@@ -28,7 +29,6 @@ namespace ark {
 using Json = ::arkmi::Json;
 
 // ---- errors and logging: "ARK <pid> <LEVEL> file:line message" -----------------
-enum LogLevel { DEBUG = 0, INFO = 1, WARN = 2, ERROR = 3 };
 LogLevel log_level();
 
 template <typename... Args>

@@ -7,20 +7,13 @@
 #include <ark/dims.hpp>
 #include <ark/error.hpp>
 #include <ark/executor.hpp>
+#include <ark/init.hpp>
+#include <ark/log.hpp>
 #include <ark/model.hpp>
+#include <ark/model_ref.hpp>
 #include <ark/planner.hpp>
+#include <ark/random.hpp>
 #include <ark/tensor.hpp>
-#include <string>
-
-namespace ark {
-
-// Library-wide initialisation (ark/api/init.cpp): reads the environment.
-void init();
-// Seeded pseudo-random ints for test data (ark/api/random.cpp).
-void srand(int seed = -1);
-int rand();
-std::string version();
-
-}  // namespace ark
+#include <ark/version.hpp>
 
 #endif  // ARK_HPP

@@ -7,6 +7,12 @@
 // Operand values are multiples of 1/2 in [-1, 1] and K = 128, so every product sum is
 // a multiple of 1/4 below 2^9 and exact in fp16: the comparison is bit for bit.
 #include <ark/ark.hpp>
+// the single headers a program may name instead of the umbrella one
+#include <ark/init.hpp>
+#include <ark/log.hpp>
+#include <ark/model_ref.hpp>
+#include <ark/random.hpp>
+#include <ark/version.hpp>
 
 #include <cmath>
 #include <cstdint>
@@ -35,6 +41,10 @@ static int fails = 0;
 
 int main() {
     ark::init();
+    static_assert(ARK_VERSION == ARK_MAJOR * 10000 + ARK_MINOR * 100 + ARK_PATCH, "version macros");
+    EXPECT(!ark::version().empty());
+    ark::log(ark::INFO, __FILE__, __LINE__, "drop_in_executor: start");  // goes to the log stream
+    ark::log(ark::DEBUG, __FILE__, __LINE__, "below the default level: not printed");
     const int M = 256, N = 256, K = 128;
     std::vector<float> a((size_t)M * K), b((size_t)K * N);
     ark::srand(42);
