@@ -212,7 +212,7 @@ namespace arkmi {
 template <typename T>
 __global__ __launch_bounds__(kBlock) void gemv_kernel(GemvDesc d, int ntasks) {
     Slot s = block_slot(dyn_lds(), kGemvLdsBytes);
-    for (int t = blockIdx.x; t < ntasks; t += gridDim.x) gemv_task<T>(d, t, s);
+    gemv_tasks<T>(d, blockIdx.x, gridDim.x, ntasks, s);
 }
 
 }  // namespace arkmi

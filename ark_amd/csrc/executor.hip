@@ -1090,6 +1090,7 @@ struct Executor {
     int barriers_elided = 0;
     int barriers_local = 0;       // grid barriers replaced by a workgroup-local sync
     int barriers_counted = 0;     // grid barriers replaced by waits on dependency counters
+    int gemv_chains = 0;          // runs of skinny matmuls streamed as one sequence
     // Analysis only (no device): compile() stops before anything touches the GPU and keeps the
     // tables it built.  force_deps: -1 take ARKMI_DEP_COUNTERS, 0 / 1 override it.
     bool dry = false;
@@ -1100,6 +1101,9 @@ struct Executor {
     size_t dry_counters = 0;
     DevWait *d_waits = nullptr;
     int32_t *d_spans = nullptr, *d_signal = nullptr;
+    GemvSeqEntry *d_gemv_seq = nullptr;
+    std::vector<GemvSeqEntry> h_gemv_seq;  // the skinny matmuls' task sequences, per workgroup
+    std::vector<int> group_sched_step;      // schedule step of every task group
     unsigned int *d_dep_counters = nullptr;
     size_t dep_counter_bytes = 0;
     int iteration_sync = 2;       // between iterations of one command: 2 grid barrier, 1 local sync, 0 nothing
@@ -1219,6 +1223,7 @@ struct Executor {
         std::vector<DevStep> steps;
         h_groups.clear();
         h_group_fam.clear();
+        group_sched_step.clear();
         int max_slot_lds = 0;
         trace_len = 0;
         const Json &task_infos = plan.at("TaskInfos");
@@ -1371,6 +1376,7 @@ struct Executor {
                 ds.kind = STEP_TASKS;
                 ds.index = (int)h_groups.size();
                 h_groups.push_back(g);
+                group_sched_step.push_back((int)si);
             }
             dev_step_of[si] = (int)steps.size();
             steps.push_back(ds);
@@ -1579,6 +1585,86 @@ struct Executor {
         // the counters count per iteration, and a reader relies on the caches having been
         // invalidated since the previous one
         if (barriers_counted > 0) iteration_sync = 2;
+
+        // ---- skinny matmuls: every workgroup's tasks as a table; runs of them as one stream ------
+        // A skinny matmul is a few units of weights per workgroup, and adding up a column block at
+        // the end of a task takes as long as streaming them.  Matmuls that follow one another with
+        // no barrier or sync in between are therefore run as one sequence: the next one's first
+        // loads are in flight while the current one folds.  ARKMI_GEMV_CHAIN=0 turns that off
+        // (each matmul is then a sequence of its own, as it is in the one-op kernels).
+        gemv_chains = 0;
+        h_gemv_seq.clear();
+        {
+            const char *chain_env = getenv("ARKMI_GEMV_CHAIN");
+            const bool chain_on = !(chain_env && atoi(chain_env) == 0) && !trace_enabled;
+            auto is_gemv = [&](const DevTaskGroup &g) {
+                return g.op_count == 1 && ops[(size_t)g.op_begin].kind == DEV_GEMV;
+            };
+            auto chainable = [&](const DevStep &st) {
+                if (st.kind != STEP_TASKS) return false;
+                const DevTaskGroup &g = h_groups[(size_t)st.index];
+                return is_gemv(g) && g.n_waits == 0 && g.signal_begin < 0;
+            };
+            // the entries of the groups [first, first + n) for every workgroup, in group order
+            auto lay_out = [&](size_t first, size_t n, int32_t &begin, int32_t &stride) {
+                std::vector<std::vector<GemvSeqEntry>> rows((size_t)grid);
+                for (size_t gi = first; gi < first + n; ++gi) {
+                    const DevTaskGroup &g = h_groups[gi];
+                    const GemvDesc &d = ops[(size_t)g.op_begin].gemv;
+                    const auto &st = sched.steps[(size_t)group_sched_step[gi]];
+                    const int64_t U = (int64_t)d.n_blocks * d.k_units;
+                    for (int block = 0; block < grid; ++block) {
+                        int order = 0;
+                        for (int64_t id : schedule_tasks_of(sched, st, block, 0)) {
+                            const int this_order = order++;
+                            if (id < 0 || id >= d.num_tasks) continue;  // (a task beyond the partition has no units)
+                            const int64_t u0 = gemv_task_begin(id, U, d.num_tasks), u1 = gemv_task_begin(id + 1, U, d.num_tasks);
+                            if (u0 >= u1) continue;
+                            GemvSeqEntry e{};
+                            e.op = g.op_begin;
+                            e.task = (int32_t)id;
+                            e.nb = (int32_t)(u0 / d.k_units);
+                            e.ku = (int32_t)(u0 % d.k_units);
+                            e.units = (int32_t)(u1 - u0);
+                            e.trace_index = trace_enabled ? g.trace_offset + (int)((id - g.task_b) / g.task_s) : -1;
+                            e.order = this_order;
+                            rows[(size_t)block].push_back(e);
+                        }
+                    }
+                }
+                size_t longest = 0;
+                for (const auto &r : rows) longest = std::max(longest, r.size());
+                begin = (int32_t)h_gemv_seq.size();
+                stride = (int32_t)longest + 1;
+                GemvSeqEntry end{};
+                end.op = -1;
+                for (const auto &r : rows) {
+                    h_gemv_seq.insert(h_gemv_seq.end(), r.begin(), r.end());
+                    h_gemv_seq.insert(h_gemv_seq.end(), (size_t)stride - r.size(), end);
+                }
+            };
+            for (size_t gi = 0; gi < h_groups.size(); ++gi)
+                if (is_gemv(h_groups[gi])) lay_out(gi, 1, h_groups[gi].seq_begin, h_groups[gi].seq_stride);
+            for (size_t i = 0; chain_on && i < steps.size();) {
+                size_t j = i;
+                if (chainable(steps[i])) {
+                    const int dtype = ops[(size_t)h_groups[(size_t)steps[i].index].op_begin].gemv.dtype;
+                    for (j = i + 1; j < steps.size() && chainable(steps[j]) &&
+                                    steps[j].index == steps[j - 1].index + 1 &&
+                                    ops[(size_t)h_groups[(size_t)steps[j].index].op_begin].gemv.dtype == dtype;
+                         ++j) {
+                    }
+                    if (j - i > 1) {
+                        DevTaskGroup &head = h_groups[(size_t)steps[i].index];
+                        head.chain = (int)(j - i);
+                        for (size_t m = i + 1; m < j; ++m) h_groups[(size_t)steps[m].index].chain = -1;
+                        lay_out((size_t)steps[i].index, j - i, head.chain_begin, head.chain_stride);
+                        ++gemv_chains;
+                    }
+                }
+                i = std::max(j, i + 1);
+            }
+        }
         lds_bytes = loop_kernel_lds_reserved() + max_slot_lds;
         if (dry) {
             (void)loop_kernel_select(families, &kernel_families);
@@ -1623,6 +1709,9 @@ struct Executor {
             ARKMI_HIP(hipMalloc((void **)&d_dep_counters, dep_counter_bytes));
             ARKMI_HIP(hipMemset(d_dep_counters, 0, dep_counter_bytes));
         }
+        if (!h_gemv_seq.empty())
+            upload(h_gemv_seq.data(), h_gemv_seq.size() * sizeof(GemvSeqEntry), (void **)&d_gemv_seq);
+        prog.gemv_seq = d_gemv_seq;
         prog.waits = d_waits;
         prog.wait_spans = d_spans;
         prog.signal_map = d_signal;
@@ -1793,7 +1882,7 @@ struct Executor {
         (void)hipSetDevice(device);
         for (void *p : {(void *)arena, (void *)ctl, (void *)d_ops, (void *)d_groups, (void *)d_steps,
                         (void *)d_trace, (void *)d_clock, (void *)d_waits, (void *)d_spans, (void *)d_signal,
-                        (void *)d_dep_counters})
+                        (void *)d_dep_counters, (void *)d_gemv_seq})
             if (p) (void)hipFree(p);
         for (void *p : scratch_allocs) (void)hipFree(p);
         scratch_allocs.clear();
@@ -1803,7 +1892,7 @@ struct Executor {
         if (own_stream && stream) (void)hipStreamDestroy(stream);
         arena = nullptr; ctl = nullptr; d_ops = nullptr; d_groups = nullptr; d_steps = nullptr;
         d_trace = nullptr; d_clock = nullptr; d_waits = nullptr; d_spans = nullptr; d_signal = nullptr;
-        d_dep_counters = nullptr; mb = nullptr; ev_begin = ev_end = nullptr; stream = nullptr;
+        d_dep_counters = nullptr; d_gemv_seq = nullptr; mb = nullptr; ev_begin = ev_end = nullptr; stream = nullptr;
         destroyed = true;
     }
 
@@ -2015,6 +2104,7 @@ int arkmi_exec_info(arkmi_exec *h, arkmi_exec_info_t *out) {
         out->barriers_local = h->ex.barriers_local;
         out->iteration_sync = h->ex.iteration_sync;
         out->barriers_counted = h->ex.barriers_counted;
+        out->gemv_chains = h->ex.gemv_chains;
     });
 }
 
@@ -2134,6 +2224,7 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
         out["BarriersElided"] = (long long)ex.barriers_elided;
         out["BarriersLocal"] = (long long)ex.barriers_local;
         out["BarriersCounted"] = (long long)ex.barriers_counted;
+        out["GemvChains"] = (long long)ex.gemv_chains;
         out["IterationSync"] = (long long)ex.iteration_sync;
         out["NumCounters"] = (long long)ex.dry_counters;
         Json steps = Json::array();
@@ -2150,6 +2241,7 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
                 j["Kind"] = "Tasks";
                 j["Group"] = (long long)st.index;
                 j["NumTasks"] = (long long)n_tasks;
+                j["Chain"] = (long long)g.chain;
                 Json waits = Json::array();
                 for (int w = 0; w < g.n_waits; ++w) {
                     const arkmi::DevWait &dw = ex.dry_waits[(size_t)(g.wait_begin + w)];

@@ -106,17 +106,37 @@ inline size_t gemv_partition(GemvDesc &d, int tasks) {
            (size_t)d.n_blocks * d.max_parts * d.m * kGemvCols * sizeof(float);
 }
 
-template <typename T>
-__device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slot &s) {
-    const int tid = s.tid, lane = tid & 63, wave = tid >> 6;
-    const int64_t U = (int64_t)d.n_blocks * d.k_units;
-    const int u_begin = (int)gemv_task_begin(task, U, d.num_tasks);
-    const int u_end = (int)gemv_task_begin(task + 1, U, d.num_tasks);
-    if (u_begin >= u_end) return;
+// One task of a workgroup's sequence of skinny-matmul tasks, as the host lays it out for the
+// loop kernel: which op, which task of it, and the units of that task (column block and K-chunk
+// of the first one, how many).  `op < 0` ends the sequence.
+struct GemvSeqEntry {
+    int32_t op;
+    int32_t task;
+    int32_t nb, ku;       // first unit: column block, K-chunk inside it
+    int32_t units;        // > 0
+    int32_t trace_index;  // where the task's trace record goes, -1: nowhere
+    int32_t order;        // the task's number on this workgroup within its group
+    int32_t pad_;
+};
 
-    gptr<const T> W = as_global(static_cast<const T *>(d.w));
-    gptr<const T> X = as_global(static_cast<const T *>(d.x));
-    gptr<T> Y = as_global(static_cast<T *>(d.y));
+// Where a workgroup is in the units it has to stream.  Two of these walk the same sequence,
+// the one that issues loads two units ahead of the one that multiplies.
+struct GemvCursor {
+    GemvDesc d;
+    int index = 0;       // of the next task in the sequence
+    int task = 0;
+    int nb = 0, ku = 0;  // the current unit
+    int left = 0;        // units of the current task still to go, this one included; 0: the end
+    bool from_zero = false;  // the current column-block segment began at the block's first K-chunk
+};
+
+// Streams the units of a sequence of skinny-matmul tasks through one workgroup.
+// `source(i, d, task, nb, ku, units)` describes the i-th task of the sequence (false: there is
+// none).  Between two tasks the loads never stop: while the last column block of a task is added
+// up and stored, the first two units of the next task are already in flight.
+template <typename T, typename Source>
+__device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
+    const int tid = s.tid, lane = tid & 63, wave = tid >> 6;
 
     lds_i32 *flag = (lds_i32 *)s.lds;
     const lds_ptr wlds = s.lds + 64 + wave * kGemvWaveBytes;
@@ -128,14 +148,29 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
 
     // X fragment (B operand): lane holds x[m = lane%16][k = k0 + (lane/16)*4 .. +3]
     const int xm = lane & 15, xk = (lane >> 4) * 4;
-    const bool x_ok = xm < d.m;
-    gptr<const T> xsrc = X + (int64_t)xm * d.ldx + xk;
 
     // W^T fragment (A operand) through the transposing read: inside each block
     // of 16 lanes (one k-group of 4), lane i supplies the address of 4
     // consecutive n at row i/4 and receives 4 consecutive k of column i
     const int i16 = lane & 15;
     const int wfrag = ((lane >> 4) * 4 + (i16 >> 2)) * kGemvRowBytes + (i16 & 3) * 8;
+
+    auto seek = [&](GemvCursor &c) {  // to the first unit of the next task
+        if (!source(c.index, c.d, c.task, c.nb, c.ku, c.left)) {
+            c.left = 0;
+            return;
+        }
+        ++c.index;
+        c.from_zero = (c.ku == 0);
+    };
+    auto advance = [&](GemvCursor &c) {
+        if (--c.left <= 0) {
+            seek(c);
+        } else if (++c.ku == c.d.k_units) {
+            c.ku = 0;
+            ++c.nb;
+        }
+    };
 
     constexpr int NG = kGemvCols / 16;  // 16 MFMA tiles per wave
     f32x4 acc[NG];
@@ -146,8 +181,11 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
     // two units are kept in flight per wave (16 KB), in two register sets
     u32x4 stage_a[NLD], stage_b[NLD];
     u32x2 x_a, x_b;
-    auto gload = [&](int u, u32x4(&stage)[NLD], u32x2 &xf) {
-        const int nb = u / d.k_units, ku = u - nb * d.k_units;
+    auto gload = [&](const GemvCursor &c, u32x4(&stage)[NLD], u32x2 &xf) {
+        const GemvDesc &d = c.d;
+        gptr<const T> W = as_global(static_cast<const T *>(d.w));
+        gptr<const T> xsrc = as_global(static_cast<const T *>(d.x)) + (int64_t)xm * d.ldx + xk;
+        const int nb = c.nb, ku = c.ku;
         const int k0 = ku * kGemvUnitK + wave * kGemvStepK;  // this wave's first row
         // Loads are unconditional: a column past N is clamped to the last
         // vector of the row (its products are never stored) and a row past K to
@@ -164,7 +202,7 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
             stage[i] = v;
         }
         u32x2 xv{0u, 0u};
-        if (x_ok) {
+        if (xm < d.m) {
             // the last k-group of a ragged K may reach past the row: fetch by element
             if (k0 + xk + 4 <= d.k) {
                 xv = *(const ARKMI_GLOBAL u32x2 *)(xsrc + k0);
@@ -179,19 +217,29 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
         xf = xv;
     };
 
-    gload(u_begin, stage_a, x_a);
-    if (u_begin + 1 < u_end) gload(u_begin + 1, stage_b, x_b);
-    int seg_begin = u_begin;  // first unit of the current column block's segment
+    GemvCursor L, C;  // loads run two units ahead of the products
+    seek(L);
+    if (L.left <= 0) return;
+    C = L;
+    gload(L, stage_a, x_a);
+    advance(L);
+    if (L.left > 0) {
+        gload(L, stage_b, x_b);
+        advance(L);
+    }
     // One unit: park it in LDS, refill its register set with the unit after
     // next, multiply, and fold the tiles when the column block is left.
-    auto consume = [&](int u, u32x4(&stage)[NLD], u32x2 &xf) {
+    auto consume = [&](u32x4(&stage)[NLD], u32x2 &xf) {
         // only this wave touches its window, and LDS serves one wave's requests
         // in order, so a wave-level fence is enough
 #pragma unroll
         for (int i = 0; i < NLD; ++i)
             *(lds_u32x4 *)(wlds + wdst + 2 * i * kGemvRowBytes) = stage[i];
         const u32x2 xcur = xf;
-        if (u + 2 < u_end) gload(u + 2, stage, xf);
+        if (L.left > 0) {
+            gload(L, stage, xf);
+            advance(L);
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -212,68 +260,90 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        const int nb = u / d.k_units;
-        const bool block_ends = (u + 1 == (nb + 1) * d.k_units);
-        if (!block_ends && u + 1 < u_end) return;
+        const GemvDesc &d = C.d;
+        const int task = C.task, nb = C.nb;
+        const bool block_ends = (C.ku + 1 == d.k_units);
+        if (!block_ends && C.left > 1) return;
 
         // ---- leaving column block nb: add the 8 waves' tiles through LDS ----------------
         // accumulator layout of 16x16x16: lane holds column (lane%16) = m and rows
         // 4*(lane/16) + r = n inside the tile
+        gptr<T> Y = as_global(static_cast<T *>(d.y));
         s.sync();  // every wave is done with its staging window
         {
             lds_f32 *red = (lds_f32 *)wlds;
             const int m = lane & 15, nq = (lane >> 4) * 4;
+            const bool live = m < d.m;  // (the other lanes hold products of X's zero padding)
 #pragma unroll
             for (int g = 0; g < NG; ++g) {
-                *(lds_f32x4 *)(red + m * kGemvRedPitch + g * 16 + nq) = acc[g];
+                if (live) *(lds_f32x4 *)(red + m * kGemvRedPitch + g * 16 + nq) = acc[g];
                 acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
             }
         }
         s.sync();
-        const int n_local = tid & (kGemvCols - 1);
-        const int col = nb * kGemvCols + n_local;
-        float sums[8];
+        // a thread adds up four consecutive columns of one row (a wave one row of the block, the
+        // workgroup eight rows at a time) over the eight waves' windows
+        const int c4 = (tid & 63) * 4, mrow = tid >> 6;
+        const int col = nb * kGemvCols + c4;  // n is a multiple of 8: col < n means col + 4 <= n
+        f32x4 sums[2];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int m = (tid >> 8) + 2 * j;
-            float v = 0.f;
+        for (int pass = 0; pass < 2; ++pass) {
+            const int m = mrow + 8 * pass;
+            f32x4 v{0.f, 0.f, 0.f, 0.f};
             if (m < d.m) {
 #pragma unroll
                 for (int w = 0; w < kGemvWaves; ++w)
-                    v += *(const lds_f32 *)(s.lds + 64 + w * kGemvWaveBytes +
-                                            (m * kGemvRedPitch + n_local) * 4);
+                    v += *(const lds_f32x4 *)(s.lds + 64 + w * kGemvWaveBytes + (m * kGemvRedPitch + c4) * 4);
             }
-            sums[j] = v;
-            __builtin_amdgcn_sched_barrier(0);
+            sums[pass] = v;
         }
-        const bool whole_block = (seg_begin == nb * d.k_units) && block_ends;
+        const bool vec_ok = ((d.ldy & 3) == 0) && (((uintptr_t)d.y & 7) == 0);
+        auto store_y = [&](int m, f32x4 v) {
+            gptr<T> p = Y + (int64_t)m * d.ldy + col;
+            T o[4] = {from_f32<T>(v[0]), from_f32<T>(v[1]), from_f32<T>(v[2]), from_f32<T>(v[3])};
+            if (vec_ok) {
+                u32x2 w;
+                __builtin_memcpy(&w, o, 8);
+                *(ARKMI_GLOBAL u32x2 *)p = w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) p[e] = o[e];
+            }
+        };
+        const bool whole_block = C.from_zero && block_ends;
         if (whole_block) {
             if (col < d.n) {
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int m = (tid >> 8) + 2 * j;
-                    if (m < d.m) Y[(int64_t)m * d.ldy + col] = from_f32<T>(sums[j]);
+                for (int pass = 0; pass < 2; ++pass) {
+                    const int m = mrow + 8 * pass;
+                    if (m < d.m) store_y(m, sums[pass]);
                 }
             }
         } else {
             // K of this block is shared with other tasks: partial + arrival counter.
-            // Partials travel as agent-scope relaxed atomics (write-through
-            // stores, L2-bypassing loads), so no cache-wide write-back or
-            // invalidate is needed: those are serialised per L2 and cost more
-            // than the op itself when every task issues them.  Ordering: every
-            // wave waits for its stores to be acknowledged (vmcnt 0) before the
-            // workgroup barrier, the counter is bumped after it, and the partials
-            // are read only after the counter has been seen full.
+            // Partials travel as 16-byte buffer stores and loads with the agent-scope
+            // bit (written through to memory, read past this XCD's L2), so no
+            // cache-wide write-back or invalidate is needed: those are serialised
+            // per L2 and cost more than the op itself when every task issues them.
+            // Ordering: every wave waits for its stores to be acknowledged (vmcnt 0)
+            // before the workgroup barrier, the counter is bumped after it, and the
+            // partials are read only after the counter has been seen full.
+            constexpr int kAgentScope = 16;  // cache-policy bit sc1 of the buffer instructions
+            const int64_t U = (int64_t)d.n_blocks * d.k_units;
             const int t_first = (int)gemv_task_of((int64_t)nb * d.k_units, U, d.num_tasks);
             const int t_last = (int)gemv_task_of((int64_t)(nb + 1) * d.k_units - 1, U, d.num_tasks);
             const int parts = t_last - t_first + 1;
+            const int part_bytes = d.m * kGemvCols * 4;
             float *Pb = d.partial + (int64_t)nb * d.max_parts * d.m * kGemvCols;
+            const __amdgpu_buffer_rsrc_t rsrc =
+                __builtin_amdgcn_make_buffer_rsrc(Pb, 0, d.max_parts * part_bytes, 0x00020000);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int m = (tid >> 8) + 2 * j;
+            for (int pass = 0; pass < 2; ++pass) {
+                const int m = mrow + 8 * pass;
                 if (m < d.m)
-                    __hip_atomic_store(Pb + ((int64_t)(task - t_first) * d.m + m) * kGemvCols + n_local,
-                                       sums[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sums[pass]), rsrc,
+                                                           (task - t_first) * part_bytes + (m * kGemvCols + c4) * 4,
+                                                           0, kAgentScope);
             }
             drain_stores_then_barrier();
             if (tid == 0) {
@@ -285,25 +355,25 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
             if (*flag) {
                 if (col < d.n) {
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        const int m = (tid >> 8) + 2 * j;
+                    for (int pass = 0; pass < 2; ++pass) {
+                        const int m = mrow + 8 * pass;
                         if (m < d.m) {
                             // four loads in flight per row, added in task order
-                            float v = 0.f;
+                            f32x4 v{0.f, 0.f, 0.f, 0.f};
                             for (int q0 = 0; q0 < parts; q0 += 4) {
-                                float t[4];
+                                u32x4 t[4];
 #pragma unroll
                                 for (int i = 0; i < 4; ++i)
                                     t[i] = (q0 + i < parts)
-                                               ? __hip_atomic_load(
-                                                     Pb + ((int64_t)(q0 + i) * d.m + m) * kGemvCols + n_local,
-                                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                                               : 0.f;
+                                               ? __builtin_amdgcn_raw_buffer_load_b128(
+                                                     rsrc, (q0 + i) * part_bytes + (m * kGemvCols + c4) * 4, 0,
+                                                     kAgentScope)
+                                               : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
                                 for (int i = 0; i < 4; ++i)
-                                    if (q0 + i < parts) v += t[i];
+                                    if (q0 + i < parts) v += __builtin_bit_cast(f32x4, t[i]);
                             }
-                            Y[(int64_t)m * d.ldy + col] = from_f32<T>(v);
+                            store_y(m, v);
                         }
                     }
                 }
@@ -312,17 +382,34 @@ __device__ __forceinline__ void gemv_task(const GemvDesc &d, int task, const Slo
             }
         }
         s.sync();  // the windows (and the flag) are reused by the next segment
-        seg_begin = u + 1;
+        C.from_zero = block_ends;  // (a task that ends inside a block is followed by a new task)
     };
-    for (int u = u_begin; u < u_end; u += 2) {
-        consume(u, stage_a, x_a);
-        if (u + 1 < u_end) consume(u + 1, stage_b, x_b);
+    for (;;) {
+        consume(stage_a, x_a);
+        advance(C);
+        if (C.left <= 0) break;
+        consume(stage_b, x_b);
+        advance(C);
+        if (C.left <= 0) break;
     }
 }
 
-__device__ __forceinline__ void gemv_dispatch(const GemvDesc &d, int task, const Slot &s) {
-    if (d.dtype == 1) gemv_task<f16>(d, task, s);
-    else gemv_task<bf16>(d, task, s);
+// The tasks first, first + stride, ... < end of one skinny matmul, as one stream.
+template <typename T>
+__device__ __forceinline__ void gemv_tasks(const GemvDesc &d, int first, int stride, int end, const Slot &s) {
+    const int64_t U = (int64_t)d.n_blocks * d.k_units;
+    gemv_stream<T>(s, [&](int i, GemvDesc &out, int &task, int &nb, int &ku, int &units) {
+        const int t = first + i * stride;
+        if (t >= end) return false;
+        // (every task has a unit: the partition never makes more tasks than units)
+        const int u_begin = (int)gemv_task_begin(t, U, d.num_tasks);
+        out = d;
+        task = t;
+        nb = u_begin / d.k_units;
+        ku = u_begin - nb * d.k_units;
+        units = (int)gemv_task_begin(t + 1, U, d.num_tasks) - u_begin;
+        return units > 0;
+    });
 }
 
 }  // namespace arkmi

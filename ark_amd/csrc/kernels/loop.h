@@ -62,7 +62,17 @@ struct DevTaskGroup {
     // As a producer: task index i completes row block signal_map[signal_begin + i] and adds one
     // to counter signal_base + that block; signal_begin < 0: the group signals nothing.
     int32_t signal_begin, signal_base;
-    int32_t pad_[1];
+    // A group of skinny-matmul tasks runs from a table the host lays out, LoopProgram::gemv_seq:
+    // workgroup b's tasks of the group, in order, are the entries from seq_begin + b * seq_stride
+    // up to the first one with op < 0.  Groups that follow one another with nothing to wait for
+    // in between are streamed as one sequence by the loop kernel (the next matmul's weights are
+    // on their way while the current one adds up its tiles): chain = n > 1 on the first group
+    // of such a run (the groups gi .. gi + n - 1), whose chain_begin / chain_stride name the
+    // sequence of the whole run, and chain = -1 on the others, which the loop kernel skips.
+    // The one-op kernels run every group from its own table.
+    int32_t chain;
+    int32_t seq_begin, seq_stride;
+    int32_t chain_begin, chain_stride;
 };
 
 // One producer a task group waits for.
@@ -130,6 +140,7 @@ struct LoopProgram {
     const int32_t *wait_spans;
     const int32_t *signal_map;
     unsigned int *dep_counters;
+    const GemvSeqEntry *gemv_seq;  // the task sequences of the skinny matmuls, null if there are none
     int32_t num_steps;
     int32_t num_blocks;
     // what separates two iterations of the body inside one command:
@@ -149,7 +160,7 @@ struct LoopArgs {
     HostMailbox *mb;
     uint64_t idle_ticks, wait_ticks;
     int32_t one_shot_iters;  // loop kernel: > 0 runs that many iterations and returns
-    int32_t group;           // one-op kernel: the task group to run
+    int32_t group;           // one-op kernel: the task group to run; loop kernel: -1
 };
 
 // Mapped, pinned host memory shared with the kernel.

@@ -100,6 +100,7 @@ void loop_kernel_launch(const void *kernel, const LoopProgram &prog, LoopControl
     a.ctl = ctl; a.mb = mb_dev;
     a.idle_ticks = idle_ticks; a.wait_ticks = wait_ticks;
     a.one_shot_iters = one_shot_iters;
+    a.group = -1;  // all of them
     void *args[] = {&a};
     ARKMI_HIP(hipLaunchKernel(kernel, dim3(grid), dim3(threads), args, (size_t)lds_bytes, stream));
 }

@@ -403,15 +403,49 @@ ARKMI_BODY int gemm_f32_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, 
                           });
 }
 
-ARKMI_BODY int gemv_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, unsigned epoch) {
+// This workgroup's skinny-matmul tasks from the sequence at `seq` (the host's table), one after
+// the other, with the loads running on across the boundaries between tasks and between matmuls.
+template <typename T>
+__device__ __forceinline__ void gemv_sequence(KArgs ka, const GemvSeqEntry *seq, const Slot &s) {
+    gemv_stream<T>(s, [&](int i, GemvDesc &out, int &task, int &nb, int &ku, int &units) {
+        const GemvSeqEntry e = load_const(seq + i);
+        if (e.op < 0) return false;
+#ifndef ARKMI_NO_TRACE
+        TraceRecord *trace = KARG(prog.trace);
+        if (trace && e.trace_index >= 0 && s.tid == 0) {
+            TraceRecord rec{(int)blockIdx.x, 0, e.order};
+            trace[e.trace_index] = rec;
+        }
+#endif
+        out = load_const(&(KARG(prog.ops) + e.op)->gemv);
+        task = e.task;
+        nb = e.nb;
+        ku = e.ku;
+        units = e.units;
+        return true;
+    });
+}
+
+// (Skinny matmuls take no part in the dependency counters: the host keeps the barriers around
+// them, so there is nothing to wait for or to signal here.)
+ARKMI_BODY int gemv_body(KArgs ka_in, int gi_in, int t0, int tid, lds_ptr lds, unsigned epoch) {
     const KArgs ka = uniform_kargs(ka_in);
     const Slot s = body_slot(tid, lds);
-    return long_task_loop(ka, __builtin_amdgcn_readfirstlane(gi), __builtin_amdgcn_readfirstlane(t0), tid,
-                          __builtin_amdgcn_readfirstlane(epoch), s.lds - kLdsReserved, [&](const DevOp *op, int task) {
-                              const GemvDesc d = load_const(&op->gemv);
-                              gemv_dispatch(d, task, s);
-                              return task;
-                          });
+    const int gi = __builtin_amdgcn_readfirstlane(gi_in);
+    const DevTaskGroup *g = KARG(prog.groups) + gi;
+    // the loop kernel streams a run of groups from the first one; the one-op kernels (which name
+    // their group in the kernel arguments) run every group by itself
+    const bool run = KARG(group) < 0 && load_const(&g->chain) > 1;
+    const int begin = run ? load_const(&g->chain_begin) : load_const(&g->seq_begin);
+    const int stride = run ? load_const(&g->chain_stride) : load_const(&g->seq_stride);
+    const GemvSeqEntry *seq = KARG(prog.gemv_seq) + begin + (size_t)blockIdx.x * stride;
+    const int op = load_const(&seq->op);
+    if (op >= 0) {
+        // (one element type per sequence: checked on the host)
+        if (load_const(&(KARG(prog.ops) + op)->gemv.dtype) == 1) gemv_sequence<f16>(ka, seq, s);
+        else gemv_sequence<bf16>(ka, seq, s);
+    }
+    return kTasksDone;
 }
 
 ARKMI_BODY int attn_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, unsigned epoch) {
@@ -549,6 +583,18 @@ template <int FAM>
 __device__ __forceinline__ bool run_group(KArgs ka, const LoopProgram &P, int gi, unsigned epoch) {
     const TaskDeal d = deal_of(P.groups, gi);
     const DevTaskGroup &g = d.g;
+    if constexpr ((FAM & FAM_GEMV) != 0) {
+        if (KARG(group) < 0) {
+            // a skinny matmul that the first group of its run has already streamed
+            if (g.chain < 0) return true;
+            // the first group of a run: the host's table says what this workgroup does for the
+            // run, whether or not it has a task of the first matmul
+            if (g.chain > 1) {
+                const Slot s0 = body_slot(threadIdx.x, (lds_ptr)g_loop_lds + kLdsReserved);
+                return run_long_tasks<FAM, DEV_GEMV>(ka, gi, s0, epoch);
+            }
+        }
+    }
     if (!d.mine) return true;
     const int slot_threads = g.slot_warps * kWave;
     const int k = threadIdx.x / slot_threads;

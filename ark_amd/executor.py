@@ -26,7 +26,8 @@ class ExecInfo(ctypes.Structure):
                 ("compiled", ctypes.c_int), ("launched", ctypes.c_int),
                 ("destroyed", ctypes.c_int), ("loop_mode", ctypes.c_int),
                 ("iterations_done", ctypes.c_int), ("barriers_local", ctypes.c_int),
-                ("iteration_sync", ctypes.c_int), ("barriers_counted", ctypes.c_int)]
+                ("iteration_sync", ctypes.c_int), ("barriers_counted", ctypes.c_int),
+                ("gemv_chains", ctypes.c_int)]
 
 
 def _i64(v):

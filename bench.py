@@ -309,6 +309,79 @@ def config_c5(torch, np, Model, Executor, llama, inp, cpu):
     return out
 
 
+def timeline(torch, np, Model, Executor, llama, prng, which):
+    """Per-step workgroup clocks of one configuration's plan in the loop kernel (text, for the
+    profile summaries): every workgroup reads the clock when it enters a step, so a step's
+    duration per workgroup and the spread of the entry times show where workgroups wait."""
+    import json as _json
+    import os as _os
+    from ark_amd import plan_schedule
+    inp = Inputs(torch, prng, which.upper())
+    cases = []
+    if which == "c4":
+        for bsz in (1, 8):
+            m = Model()
+            feeds = []
+            for name, k, n in [("W_qkv", 4096, 12288), ("W_o", 4096, 4096), ("W_gate_up", 4096, 22016), ("W_down", 11008, 4096)]:
+                tx, tw = m.tensor([bsz, k], "bf16"), m.tensor([k, n], "bf16")
+                m.matmul(tx, tw)
+                feeds += [(tx, inp.normal(f"x_{name}_b{bsz}", tx.shape, torch.bfloat16)),
+                          (tw, inp.normal(name, tw.shape, torch.bfloat16, 0.02))]
+            cases.append((f"C4 batch {bsz}", m.plan(device_id=0), feeds, {}))
+    else:
+        m = Model()
+        blk = llama.TransformerBlock(m, 4096, 32, 11008, "bf16")
+        tx, tf, tm = m.tensor([1, 2048, 4096], "bf16"), m.tensor([1, 2048, 1, 128], "bf16"), m.tensor([1, 1, 2048, 2048], "bf16")
+        blk.forward(tx, tf, tm, fused=True, causal=True)
+        feeds = [(tx, inp.normal("hidden", tx.shape, torch.bfloat16)),
+                 (tf, torch.from_numpy(llama.precompute_freqs_cis(128, 2048)).cuda().bfloat16())]
+        for name, t in blk.params().items():
+            feeds.append((t, torch.ones(*t.shape, device="cuda") if name.endswith("_norm")
+                          else inp.normal(name, t.shape, torch.bfloat16, 0.02)))
+        plan = m.plan(device_id=0)
+        cases.append(("C5 fused ops with the attention op, grid barriers", plan, feeds, {}))
+        cases.append(("C5 fused ops with the attention op, dependency counters", plan, feeds, {"ARKMI_DEP_COUNTERS": "1"}))
+    for title, plan, feeds, env in cases:
+        names = {ti["Id"]: "+".join(o["Type"] for o in ti["Ops"]) for ti in _json.loads(plan)["TaskInfos"]}
+        sched = [(names[st["Args"][-1]] if st["Kind"] == "TaskSeq" else "B") for st in plan_schedule(plan)["Steps"]]
+        _os.environ.update(env)
+        try:
+            ex = Executor(plan, device_id=0, trace=True).compile()
+        finally:
+            for k in env:
+                del _os.environ[k]
+        for t, x in feeds:
+            ex.tensor_write_device(t, x)
+        torch.cuda.synchronize()
+        ex.launch()
+        ex.run(10)
+        ex.wait()
+        t0 = time.perf_counter()
+        ex.run(20)
+        ex.wait()
+        us = (time.perf_counter() - t0) / 20 * 1e6
+        info = ex.info()
+        clk, _ = ex.read_step_clocks()
+        ex.stop()
+        clk = np.array(clk)
+        base, d = clk[:, 0].min(), np.diff(clk, axis=1)
+        print(f"{title}: {us:.1f} us per iteration with the clocks on; "
+              + ", ".join(f"{k} {info[k]}" for k in ("barriers_elided", "barriers_local", "barriers_counted",
+                                                      "iteration_sync", "gemv_chains", "kernel_families")))
+        print("  schedule: " + " | ".join(sched))
+        print("  us, over the workgroups:   time in the step min / median / max      step entered first / last")
+        for i in range(d.shape[1]):
+            print(f"  step {i:2d} {sched[i][:22]:22s} {d[:, i].min():8.2f} {np.median(d[:, i]):8.2f} {d[:, i].max():8.2f}"
+                  f"      {clk[:, i].min() - base:9.2f} {clk[:, i].max() - base:9.2f}")
+        print(f"  end of the body reached first / last {clk[:, -1].min() - base:9.2f} {clk[:, -1].max() - base:9.2f}")
+        if which == "c4":
+            # by XCD (workgroups go to the XCDs round robin): does one of them stream more slowly?
+            tot = clk[:, -1] - clk[:, 0]
+            print("  time in the body by XCD (workgroup index mod 8), median: "
+                  + "  ".join(f"{np.median(tot[x::8]):.1f}" for x in range(8)))
+        del ex
+
+
 def machine_probes(torch, prng):
     """What this GPU sustains: an MFMA-only loop (random and zero operands) and plain streams."""
     import ctypes
@@ -399,6 +472,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the other configurations (C1, C3, C4, C5)")
     ap.add_argument("--only", choices=["c1", "c3", "c4", "c5"], default=None,
                     help="run only this configuration and print its block (for profiling one configuration)")
+    ap.add_argument("--timeline", action="store_true",
+                    help="with --only c4 or c5: print the per-step workgroup clocks of the plan instead (text)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU; this build has no multi-GPU path "
@@ -414,6 +489,12 @@ def main():
     info = ark_amd.device_info(0)
     cpu = not args.no_cpu_baseline
 
+    if args.timeline:
+        if args.only not in ("c4", "c5"):
+            print("--timeline needs --only c4 or --only c5", file=sys.stderr)
+            sys.exit(2)
+        timeline(torch, np, Model, Executor, llama, prng, args.only)
+        return
     if args.only:
         print(json.dumps({"only": args.only,
                           "configs": other_configs(torch, np, Model, Executor, llama, prng, cpu, only=args.only)}))

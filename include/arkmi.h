@@ -262,6 +262,7 @@ typedef struct arkmi_exec_info_t {
     int barriers_local;   /* grid barriers replaced by a workgroup-local sync */
     int iteration_sync;   /* between iterations of one run(n): 2 grid barrier, 1 workgroup-local sync, 0 nothing */
     int barriers_counted; /* grid barriers replaced by waits on per-row-block dependency counters */
+    int gemv_chains;      /* runs of consecutive skinny matmuls that the loop kernel streams as one sequence */
 } arkmi_exec_info_t;
 
 int arkmi_exec_create(int device_id, void *stream, const char *name,

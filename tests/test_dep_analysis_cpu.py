@@ -141,3 +141,37 @@ def test_analysis_rejects_what_compile_rejects():
     with pytest.raises(ArkmiError) as e:
         plan_analysis("{not json", 1)
     assert e.value.kind == "PlanError"
+
+
+def test_consecutive_skinny_matmuls_form_one_stream():
+    """Skinny matmuls that follow one another with no barrier or sync between them are marked as one
+    run (the first group carries the length, the others -1); anything in between, a dependency, or
+    an op fused into the task breaks the run."""
+    m = Model()
+    for k, n in [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]:
+        m.matmul(m.tensor([1, k], "bf16"), m.tensor([k, n], "bf16"))
+    a = plan_analysis(_plan(m), 0)
+    assert a["GemvChains"] == 1
+    assert [s["Kind"] for s in a["Steps"]] == ["Tasks"] * 4
+    assert [s["Chain"] for s in a["Steps"]] == [4, -1, -1, -1]
+
+    # y2 depends on y1: the barrier between them stays and nothing is chained
+    m = Model()
+    y1 = m.matmul(m.tensor([1, 4096], "bf16"), m.tensor([4096, 4096], "bf16"))
+    m.matmul(y1, m.tensor([4096, 4096], "bf16"))
+    a = plan_analysis(_plan(m), 0)
+    assert a["GemvChains"] == 0 and [s["Kind"] for s in a["Steps"]] == ["Tasks", "Barrier", "Tasks"]
+    assert [s["Chain"] for s in _tasks_steps(a)] == [0, 0]
+
+    # two runs separated by an elementwise op of its own
+    m = Model()
+    for _ in range(2):
+        m.matmul(m.tensor([2, 1024], "fp16"), m.tensor([1024, 512], "fp16"))
+    m.relu(m.tensor([64, 64], "fp16"))
+    for _ in range(3):
+        m.matmul(m.tensor([2, 1024], "fp16"), m.tensor([1024, 512], "fp16"))
+    # a different element type does not join the run before it
+    m.matmul(m.tensor([2, 1024], "bf16"), m.tensor([1024, 512], "bf16"))
+    a = plan_analysis(_plan(m), 0)
+    assert a["GemvChains"] == 2
+    assert [s["Chain"] for s in _tasks_steps(a)] == [2, -1, 0, 3, -1, -1, 0]

@@ -162,7 +162,7 @@ def test_decode_step_four_projections_in_one_plan(oracle, batch):
         vals[tw] = make(oracle, (k, n), dtype, seed=50 + i, dist="normal", scale=0.02)
         xs.append(tx); ws.append(tw); ys.append(mod.matmul(tx, tw))
     ex = Executor(mod.plan(device_id=0)).compile()
-    assert ex.info()["kernel_families"] == 8
+    assert ex.info()["kernel_families"] == 8 and ex.info()["gemv_chains"] == 1
     for t, a in vals.items():
         ex.tensor_write(t, a)
     ex.launch()
@@ -174,3 +174,50 @@ def test_decode_step_four_projections_in_one_plan(oracle, batch):
         cols = np.sort(np.random.default_rng(n).choice(n, 512, replace=False))
         cols[0], cols[-1] = 0, n - 1
         _sampled_columns_check(oracle, vals[tx], vals[tw], g, dtype, cols)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_consecutive_skinny_matmuls_run_as_one_stream(oracle, dtype, monkeypatch):
+    """Independent skinny matmuls that follow one another are streamed as one sequence by the loop
+    kernel (the next one's weights are loaded while the current one adds up its tiles).  Shapes with
+    ragged K and N, different row counts, few tasks (most workgroups have nothing to do for that
+    matmul) and many: every output against the oracle, and bit for bit against the same plan with
+    the matmuls run one by one (ARKMI_GEMV_CHAIN=0) and as one kernel per op."""
+    from ark_amd import Model, Executor
+    shapes = [(1, 2048, 1536), (3, 296, 264), (8, 4096, 512), (16, 1024, 8), (2, 16, 4096), (1, 11008, 1024)]
+    mod = Model()
+    vals, ys = {}, []
+    for i, (m, k, n) in enumerate(shapes):
+        tx, tw = mod.tensor([m, k], dtype), mod.tensor([k, n], dtype)
+        vals[tx] = make(oracle, (m, k), dtype, seed=60 + i, dist="normal")
+        vals[tw] = make(oracle, (k, n), dtype, seed=70 + i, dist="normal", scale=0.05)
+        ys.append((mod.matmul(tx, tw), tx, tw, k))
+    plan = mod.plan(device_id=0)
+
+    def run(separate=False):
+        ex = Executor(plan, device_id=0, loop_mode=not separate).compile()
+        info = ex.info()
+        for t, a in vals.items():
+            ex.tensor_write(t, a)
+        if separate:
+            ex.run_separate(2)
+            torch.cuda.synchronize()
+        else:
+            ex.launch()
+            ex.run(3)
+            ex.wait()
+        got = [ex.tensor_read(y) for y, _, _, _ in ys]
+        if not separate:
+            ex.stop()
+        return got, info
+
+    chained, info = run()
+    assert info["kernel_families"] == 8 and info["gemv_chains"] == 1
+    for g, (_, tx, tw, k) in zip(chained, ys):
+        _check(oracle, oracle.matmul(vals[tx], vals[tw], dtype), g, dtype, 4.0 * 0.25, k)
+    one_kernel_per_op, _ = run(separate=True)
+    monkeypatch.setenv("ARKMI_GEMV_CHAIN", "0")
+    one_by_one, info = run()
+    assert info["gemv_chains"] == 0
+    for a, b, c in zip(chained, one_by_one, one_kernel_per_op):
+        assert np.array_equal(a, b) and np.array_equal(a, c)
