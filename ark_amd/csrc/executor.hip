@@ -153,6 +153,23 @@ Schedule build_schedule(const Json &plan) {
     return sch;
 }
 
+// Cutting a run of skinny matmuls into stretches that the workgroups claim at run time: the
+// first `coarse_share` of the run's units goes into long stretches (two of them are about that
+// share of a workgroup's average load: every workgroup starts with two), the rest into short ones
+// of `fine` units, so that the spread at the end of the run is a short stretch or two.
+// ARKMI_GEMV_FINE / ARKMI_GEMV_COARSE_PERCENT override the defaults (for measurements).
+constexpr int kGemvMinStretch = 3;  // the claim protocol's look-ahead needs 3 units per stretch
+int gemv_fine_units() {
+    const char *e = getenv("ARKMI_GEMV_FINE");
+    const int v = e ? atoi(e) : 0;
+    return v >= kGemvMinStretch && v <= 1024 ? v : 3;
+}
+double gemv_coarse_share() {
+    const char *e = getenv("ARKMI_GEMV_COARSE_PERCENT");
+    const int v = e ? atoi(e) : -1;
+    return (v >= 0 && v <= 100 ? v : 85) / 100.0;
+}
+
 std::vector<int64_t> schedule_tasks_of(const Schedule &sch, const ScheduleStep &st, int block, int slot) {
     // kernel_template.in:11-27
     std::vector<int64_t> out;
@@ -359,10 +376,14 @@ DevOp lower_op(const Json &op_json, const Lowering &L, int slot_warps, int block
                         "skinny Matmul operands must start 16-byte aligned with N and row pitches % 8 == 0");
             g.dtype = a.dtype;
             const int tasks = (int)cfg.at("NumTasks").as_int();
-            const size_t ws_bytes = gemv_partition(g, tasks);
+            (void)gemv_partition(g, tasks);
             if (g.num_tasks != tasks)
                 ARK_ERR(PlanError, "a skinny Matmul of ", (int64_t)g.n_blocks * g.k_units,
                         " units cannot be dealt to ", tasks, " tasks");
+            // room for the partial tiles of the finest cut the executor may choose for the block
+            g.max_parts = std::max(g.max_parts, std::max(1, g.k_units / kGemvMinStretch));
+            const size_t ws_bytes = gemv_counter_bytes(g.n_blocks) +
+                                    (size_t)g.n_blocks * g.max_parts * g.m * kGemvCols * sizeof(float);
             char *ws = static_cast<char *>(L.scratch(ws_bytes));
             g.counters = reinterpret_cast<unsigned int *>(ws);
             g.partial = reinterpret_cast<float *>(ws + gemv_counter_bytes(g.n_blocks));
@@ -1102,6 +1123,9 @@ struct Executor {
     DevWait *d_waits = nullptr;
     int32_t *d_spans = nullptr, *d_signal = nullptr;
     GemvSeqEntry *d_gemv_seq = nullptr;
+    unsigned int *d_gemv_claims = nullptr;
+    size_t gemv_claim_bytes = 0;
+    int gemv_claimed = 0;                   // skinny matmuls (or runs of them) whose stretches are claimed at run time
     std::vector<GemvSeqEntry> h_gemv_seq;  // the skinny matmuls' task sequences, per workgroup
     std::vector<int> group_sched_step;      // schedule step of every task group
     unsigned int *d_dep_counters = nullptr;
@@ -1586,17 +1610,26 @@ struct Executor {
         // invalidated since the previous one
         if (barriers_counted > 0) iteration_sync = 2;
 
-        // ---- skinny matmuls: every workgroup's tasks as a table; runs of them as one stream ------
-        // A skinny matmul is a few units of weights per workgroup, and adding up a column block at
-        // the end of a task takes as long as streaming them.  Matmuls that follow one another with
-        // no barrier or sync in between are therefore run as one sequence: the next one's first
-        // loads are in flight while the current one folds.  ARKMI_GEMV_CHAIN=0 turns that off
-        // (each matmul is then a sequence of its own, as it is in the one-op kernels).
+        // ---- skinny matmuls: stretches, who streams which, runs of matmuls as one stream ----------
+        // A workgroup streams stretches of consecutive units of one column block and folds at the
+        // end of each (across the waves, then with the block's other stretches through partial
+        // tiles in the order of the parts, so the result does not depend on who streamed what).
+        // The one-op kernels run the plan's tasks on the plan's workgroups: a task's contiguous
+        // range of units, cut at the column-block boundaries.  The loop kernel
+        //  * runs matmuls that follow one another with no barrier or sync in between as one
+        //    sequence: the next one's first loads are in flight while the current one folds
+        //    (ARKMI_GEMV_CHAIN=0: every matmul by itself);
+        //  * lets the workgroups claim stretches as they get free: a workgroup's share of the HBM bandwidth varies by tens of percent
+        //    over a step, and with fixed shares the slowest one sets the time.  The run is then
+        //    cut into long stretches first and short ones at the end (gemv_coarse_share)
+        //    (ARKMI_GEMV_CLAIM=0: the tasks' fixed shares).
         gemv_chains = 0;
+        gemv_claimed = 0;
         h_gemv_seq.clear();
         {
-            const char *chain_env = getenv("ARKMI_GEMV_CHAIN");
+            const char *chain_env = getenv("ARKMI_GEMV_CHAIN"), *claim_env = getenv("ARKMI_GEMV_CLAIM");
             const bool chain_on = !(chain_env && atoi(chain_env) == 0) && !trace_enabled;
+            const bool claim_on = !(claim_env && atoi(claim_env) == 0) && !trace_enabled;
             auto is_gemv = [&](const DevTaskGroup &g) {
                 return g.op_count == 1 && ops[(size_t)g.op_begin].kind == DEV_GEMV;
             };
@@ -1605,30 +1638,37 @@ struct Executor {
                 const DevTaskGroup &g = h_groups[(size_t)st.index];
                 return is_gemv(g) && g.n_waits == 0 && g.signal_begin < 0;
             };
-            // the entries of the groups [first, first + n) for every workgroup, in group order
+            // fixed shares: the tasks of the groups [first, first + n) on the plan's workgroups,
+            // per workgroup in group order
             auto lay_out = [&](size_t first, size_t n, int32_t &begin, int32_t &stride) {
                 std::vector<std::vector<GemvSeqEntry>> rows((size_t)grid);
                 for (size_t gi = first; gi < first + n; ++gi) {
                     const DevTaskGroup &g = h_groups[gi];
                     const GemvDesc &d = ops[(size_t)g.op_begin].gemv;
                     const auto &st = sched.steps[(size_t)group_sched_step[gi]];
-                    const int64_t U = (int64_t)d.n_blocks * d.k_units;
+                    const int64_t U = (int64_t)d.n_blocks * d.k_units, T = d.num_tasks;
                     for (int block = 0; block < grid; ++block) {
                         int order = 0;
                         for (int64_t id : schedule_tasks_of(sched, st, block, 0)) {
                             const int this_order = order++;
-                            if (id < 0 || id >= d.num_tasks) continue;  // (a task beyond the partition has no units)
-                            const int64_t u0 = gemv_task_begin(id, U, d.num_tasks), u1 = gemv_task_begin(id + 1, U, d.num_tasks);
-                            if (u0 >= u1) continue;
-                            GemvSeqEntry e{};
-                            e.op = g.op_begin;
-                            e.task = (int32_t)id;
-                            e.nb = (int32_t)(u0 / d.k_units);
-                            e.ku = (int32_t)(u0 % d.k_units);
-                            e.units = (int32_t)(u1 - u0);
-                            e.trace_index = trace_enabled ? g.trace_offset + (int)((id - g.task_b) / g.task_s) : -1;
-                            e.order = this_order;
-                            rows[(size_t)block].push_back(e);
+                            if (id < 0 || id >= T) continue;  // (a task beyond the partition has no units)
+                            const int64_t u1 = gemv_task_begin(id + 1, U, T);
+                            for (int64_t u = gemv_task_begin(id, U, T); u < u1;) {
+                                const int64_t nb = u / d.k_units, ku = u % d.k_units;
+                                const int64_t t_first = gemv_task_of(nb * d.k_units, U, T);
+                                const int64_t t_last = gemv_task_of((nb + 1) * d.k_units - 1, U, T);
+                                GemvSeqEntry e{};
+                                e.op = g.op_begin;
+                                e.nb = (int32_t)nb;
+                                e.ku = (int32_t)ku;
+                                e.units = (int32_t)std::min<int64_t>(u1 - u, d.k_units - ku);
+                                e.part = (int32_t)(id - t_first);
+                                e.parts = (int32_t)(t_last - t_first + 1);
+                                e.trace_index = trace_enabled ? g.trace_offset + (int)((id - g.task_b) / g.task_s) : -1;
+                                e.order = this_order;
+                                rows[(size_t)block].push_back(e);
+                                u += e.units;
+                            }
                         }
                     }
                 }
@@ -1643,8 +1683,60 @@ struct Executor {
                     h_gemv_seq.insert(h_gemv_seq.end(), (size_t)stride - r.size(), end);
                 }
             };
-            for (size_t gi = 0; gi < h_groups.size(); ++gi)
-                if (is_gemv(h_groups[gi])) lay_out(gi, 1, h_groups[gi].seq_begin, h_groups[gi].seq_stride);
+            // claimed at run time: possible when every column block has the 3 units a stretch needs
+            // (the claim protocol's look-ahead) and the plan's barriers span the grid
+            // (every workgroup of the grid then streams for the matmul, whatever processors the
+            // plan names for it; a barrier over part of the grid would not wait for all of them)
+            bool whole_grid_barriers = true;
+            for (const DevStep &st : steps)  // (the barriers that are left)
+                if (st.kind == STEP_BARRIER && st.count != grid) whole_grid_barriers = false;
+            auto claimable = [&](size_t first, size_t n) {
+                if (!claim_on || !whole_grid_barriers) return false;
+                for (size_t gi = first; gi < first + n; ++gi)
+                    if (ops[(size_t)h_groups[gi].op_begin].gemv.k_units < kGemvMinStretch) return false;
+                return true;
+            };
+            auto lay_out_shared = [&](size_t first, size_t n, DevTaskGroup &head) {
+                int64_t total = 0, done = 0;
+                for (size_t gi = first; gi < first + n; ++gi) {
+                    const GemvDesc &d = ops[(size_t)h_groups[gi].op_begin].gemv;
+                    total += (int64_t)d.n_blocks * d.k_units;
+                }
+                const int fine = gemv_fine_units();
+                const double share = gemv_coarse_share();
+                const int coarse = std::max(fine, (int)std::llround(share * (double)total / (2.0 * grid)));
+                head.run_begin = (int32_t)h_gemv_seq.size();
+                for (size_t gi = first; gi < first + n; ++gi) {
+                    const DevTaskGroup &g = h_groups[gi];
+                    const GemvDesc &d = ops[(size_t)g.op_begin].gemv;
+                    for (int nb = 0; nb < d.n_blocks; ++nb, done += d.k_units) {
+                        const int want = (double)done < share * (double)total ? coarse : fine;
+                        const int parts = std::max(1, std::min((d.k_units + want / 2) / want, d.k_units / kGemvMinStretch));
+                        for (int p = 0; p < parts; ++p) {
+                            GemvSeqEntry e{};
+                            e.op = g.op_begin;
+                            e.nb = nb;
+                            e.ku = (int32_t)((int64_t)p * d.k_units / parts);
+                            e.units = (int32_t)((int64_t)(p + 1) * d.k_units / parts) - e.ku;
+                            e.part = p;
+                            e.parts = parts;
+                            e.trace_index = -1;
+                            h_gemv_seq.push_back(e);
+                        }
+                    }
+                }
+                head.run_stride = (int32_t)h_gemv_seq.size() - head.run_begin;
+                head.claim = gemv_claimed++;
+            };
+            for (size_t gi = 0; gi < h_groups.size(); ++gi) {
+                DevTaskGroup &g = h_groups[gi];
+                g.claim = -1;
+                if (!is_gemv(g)) continue;
+                lay_out(gi, 1, g.seq_begin, g.seq_stride);
+                g.run_begin = g.seq_begin;
+                g.run_stride = g.seq_stride;
+            }
+            std::vector<char> in_run(h_groups.size(), 0);
             for (size_t i = 0; chain_on && i < steps.size();) {
                 size_t j = i;
                 if (chainable(steps[i])) {
@@ -1655,16 +1747,23 @@ struct Executor {
                          ++j) {
                     }
                     if (j - i > 1) {
-                        DevTaskGroup &head = h_groups[(size_t)steps[i].index];
-                        head.chain = (int)(j - i);
-                        for (size_t m = i + 1; m < j; ++m) h_groups[(size_t)steps[m].index].chain = -1;
-                        lay_out((size_t)steps[i].index, j - i, head.chain_begin, head.chain_stride);
+                        const size_t first = (size_t)steps[i].index, n = j - i;
+                        DevTaskGroup &head = h_groups[first];
+                        head.chain = (int)n;
+                        for (size_t m = 1; m < n; ++m) h_groups[first + m].chain = -1;
+                        for (size_t m = 0; m < n; ++m) in_run[first + m] = 1;
+                        if (claimable(first, n)) lay_out_shared(first, n, head);
+                        else lay_out(first, n, head.run_begin, head.run_stride);
                         ++gemv_chains;
                     }
                 }
                 i = std::max(j, i + 1);
             }
+            for (size_t gi = 0; gi < h_groups.size(); ++gi)
+                if (is_gemv(h_groups[gi]) && !in_run[gi] && claimable(gi, 1)) lay_out_shared(gi, 1, h_groups[gi]);
         }
+        // claimed stretches are counted per iteration: iterations must not overlap
+        if (gemv_claimed > 0) iteration_sync = 2;
         lds_bytes = loop_kernel_lds_reserved() + max_slot_lds;
         if (dry) {
             (void)loop_kernel_select(families, &kernel_families);
@@ -1712,6 +1811,12 @@ struct Executor {
         if (!h_gemv_seq.empty())
             upload(h_gemv_seq.data(), h_gemv_seq.size() * sizeof(GemvSeqEntry), (void **)&d_gemv_seq);
         prog.gemv_seq = d_gemv_seq;
+        if (gemv_claimed > 0) {
+            gemv_claim_bytes = (size_t)gemv_claimed * 2 * kDepStride * sizeof(unsigned int);
+            ARKMI_HIP(hipMalloc((void **)&d_gemv_claims, gemv_claim_bytes));
+            ARKMI_HIP(hipMemset(d_gemv_claims, 0, gemv_claim_bytes));
+        }
+        prog.gemv_claims = d_gemv_claims;
         prog.waits = d_waits;
         prog.wait_spans = d_spans;
         prog.signal_map = d_signal;
@@ -1747,6 +1852,7 @@ struct Executor {
         // control block and mailbox start from zero on every kernel launch
         ARKMI_HIP(hipMemsetAsync(ctl, 0, sizeof(LoopControl), stream));
         if (d_dep_counters) ARKMI_HIP(hipMemsetAsync(d_dep_counters, 0, dep_counter_bytes, stream));
+        if (d_gemv_claims) ARKMI_HIP(hipMemsetAsync(d_gemv_claims, 0, gemv_claim_bytes, stream));
         mb->status = MB_OK;
         mb->alive = 1;
         loop_kernel_launch(kernel, prog, ctl, mb_dev, grid, threads, lds_bytes, 0, idle_ticks, wait_ticks, stream);
@@ -1788,6 +1894,7 @@ struct Executor {
         } else {
             ARKMI_HIP(hipMemsetAsync(ctl, 0, sizeof(LoopControl), stream));
             if (d_dep_counters) ARKMI_HIP(hipMemsetAsync(d_dep_counters, 0, dep_counter_bytes, stream));
+            if (d_gemv_claims) ARKMI_HIP(hipMemsetAsync(d_gemv_claims, 0, gemv_claim_bytes, stream));
             loop_kernel_launch(kernel, prog, ctl, mb_dev, grid, threads, lds_bytes, iter, idle_ticks, wait_ticks,
                                stream);
         }
@@ -1882,7 +1989,7 @@ struct Executor {
         (void)hipSetDevice(device);
         for (void *p : {(void *)arena, (void *)ctl, (void *)d_ops, (void *)d_groups, (void *)d_steps,
                         (void *)d_trace, (void *)d_clock, (void *)d_waits, (void *)d_spans, (void *)d_signal,
-                        (void *)d_dep_counters, (void *)d_gemv_seq})
+                        (void *)d_dep_counters, (void *)d_gemv_seq, (void *)d_gemv_claims})
             if (p) (void)hipFree(p);
         for (void *p : scratch_allocs) (void)hipFree(p);
         scratch_allocs.clear();
@@ -1892,7 +1999,7 @@ struct Executor {
         if (own_stream && stream) (void)hipStreamDestroy(stream);
         arena = nullptr; ctl = nullptr; d_ops = nullptr; d_groups = nullptr; d_steps = nullptr;
         d_trace = nullptr; d_clock = nullptr; d_waits = nullptr; d_spans = nullptr; d_signal = nullptr;
-        d_dep_counters = nullptr; d_gemv_seq = nullptr; mb = nullptr; ev_begin = ev_end = nullptr; stream = nullptr;
+        d_dep_counters = nullptr; d_gemv_seq = nullptr; d_gemv_claims = nullptr; mb = nullptr; ev_begin = ev_end = nullptr; stream = nullptr;
         destroyed = true;
     }
 
@@ -2105,6 +2212,7 @@ int arkmi_exec_info(arkmi_exec *h, arkmi_exec_info_t *out) {
         out->iteration_sync = h->ex.iteration_sync;
         out->barriers_counted = h->ex.barriers_counted;
         out->gemv_chains = h->ex.gemv_chains;
+        out->gemv_claimed = h->ex.gemv_claimed;
     });
 }
 
@@ -2225,6 +2333,7 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
         out["BarriersLocal"] = (long long)ex.barriers_local;
         out["BarriersCounted"] = (long long)ex.barriers_counted;
         out["GemvChains"] = (long long)ex.gemv_chains;
+        out["GemvClaimed"] = (long long)ex.gemv_claimed;
         out["IterationSync"] = (long long)ex.iteration_sync;
         out["NumCounters"] = (long long)ex.dry_counters;
         Json steps = Json::array();
@@ -2242,6 +2351,7 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
                 j["Group"] = (long long)st.index;
                 j["NumTasks"] = (long long)n_tasks;
                 j["Chain"] = (long long)g.chain;
+                j["Claimed"] = g.claim >= 0;
                 Json waits = Json::array();
                 for (int w = 0; w < g.n_waits; ++w) {
                     const arkmi::DevWait &dw = ex.dry_waits[(size_t)(g.wait_begin + w)];

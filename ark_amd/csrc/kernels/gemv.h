@@ -14,15 +14,17 @@
 // staging registers for no gain in a kernel that waits on HBM.)
 //
 // Work is cut stream-K style.  A unit is 256 columns x 128 rows of W (16 rows
-// per wave, one MFMA step); units are numbered column block by column block,
-// K-chunks consecutive inside a block, and task t of T owns the contiguous
-// range [t*U/T, (t+1)*U/T).  With T = the number of CUs every CU streams the
-// same number of bytes (+-1 unit) whatever the shape.  A task walks its
-// range with the next unit's loads always in flight; when it leaves a column
-// block the 8 waves add their tiles through LDS and either store Y (the task
-// covered the block's whole K) or store an fp32 partial and count arrivals in
-// an HBM-resident counter; the task that arrives last adds the partials in
-// task order (so the result does not depend on arrival order) and stores Y.
+// per wave, one MFMA step).  A workgroup streams stretches of consecutive units
+// of one column block, the next unit's loads always in flight, also across the
+// end of a stretch; at the end of a stretch the 8 waves add their tiles through
+// LDS and either store Y (the stretch covered the block's whole K) or store an
+// fp32 partial and count arrivals in an HBM-resident counter; the workgroup that
+// arrives last adds the partials in the order of the parts (so the result does
+// not depend on arrival order) and stores Y.  Who streams which stretch is the
+// caller's matter (`Source`): the stand-alone op deals the units to T tasks in
+// contiguous ranges, so with T = the number of CUs every CU streams the same
+// number of bytes (+-1 unit) whatever the shape; the loop kernel works from the
+// host's tables, or lets the workgroups claim stretches as they get free.
 //
 // The reference runs this shape through its general GEMM
 // (ark/include/kernels/matmul.h:36-115) with a 128-row tile, 127/128 of it
@@ -106,36 +108,37 @@ inline size_t gemv_partition(GemvDesc &d, int tasks) {
            (size_t)d.n_blocks * d.max_parts * d.m * kGemvCols * sizeof(float);
 }
 
-// One task of a workgroup's sequence of skinny-matmul tasks, as the host lays it out for the
-// loop kernel: which op, which task of it, and the units of that task (column block and K-chunk
-// of the first one, how many).  `op < 0` ends the sequence.
+// A stretch of consecutive units inside one column block: what a workgroup streams in one go and
+// folds at the end.  The host cuts every skinny matmul of a plan into these and lays out who
+// streams which.  `op < 0` ends a sequence.
 struct GemvSeqEntry {
     int32_t op;
-    int32_t task;
     int32_t nb, ku;       // first unit: column block, K-chunk inside it
-    int32_t units;        // > 0
-    int32_t trace_index;  // where the task's trace record goes, -1: nowhere
-    int32_t order;        // the task's number on this workgroup within its group
-    int32_t pad_;
+    int32_t units;        // > 0, all inside block nb
+    int32_t part, parts;  // the block's K is covered by `parts` stretches; this is number `part`
+    int32_t trace_index;  // where the trace record of the stretch's task goes, -1: nowhere
+    int32_t order;        // the task's number on its workgroup within its group
 };
 
-// Where a workgroup is in the units it has to stream.  Two of these walk the same sequence,
-// the one that issues loads two units ahead of the one that multiplies.
+// Where a workgroup is in the units it has to stream.  Two of these walk the same sequence of
+// stretches, the one that issues loads two units ahead of the one that multiplies.  `Source`
+// hands out the stretches: `next(d, nb, ku, units, part, parts)` (false at the end); the fold at
+// the end of a stretch calls its `fold_begins(tid)` and `fold_ends(tid)`.
+template <typename Source>
 struct GemvCursor {
+    Source src;
     GemvDesc d;
-    int index = 0;       // of the next task in the sequence
-    int task = 0;
     int nb = 0, ku = 0;  // the current unit
-    int left = 0;        // units of the current task still to go, this one included; 0: the end
-    bool from_zero = false;  // the current column-block segment began at the block's first K-chunk
+    int left = 0;        // units of the current stretch still to go, this one included; 0: the end
+    int part = 0, parts = 1;
+    __device__ __forceinline__ explicit GemvCursor(const Source &s) : src(s) {}
 };
 
-// Streams the units of a sequence of skinny-matmul tasks through one workgroup.
-// `source(i, d, task, nb, ku, units)` describes the i-th task of the sequence (false: there is
-// none).  Between two tasks the loads never stop: while the last column block of a task is added
-// up and stored, the first two units of the next task are already in flight.
+// Streams a sequence of stretches through one workgroup.  Between two stretches the loads never
+// stop: while one is added up across the waves and stored, the first two units of the next one
+// (of the same matmul or the next) are already in flight.
 template <typename T, typename Source>
-__device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
+__device__ __forceinline__ void gemv_stream(const Slot &s, const Source &source) {
     const int tid = s.tid, lane = tid & 63, wave = tid >> 6;
 
     lds_i32 *flag = (lds_i32 *)s.lds;
@@ -155,21 +158,13 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
     const int i16 = lane & 15;
     const int wfrag = ((lane >> 4) * 4 + (i16 >> 2)) * kGemvRowBytes + (i16 & 3) * 8;
 
-    auto seek = [&](GemvCursor &c) {  // to the first unit of the next task
-        if (!source(c.index, c.d, c.task, c.nb, c.ku, c.left)) {
-            c.left = 0;
-            return;
-        }
-        ++c.index;
-        c.from_zero = (c.ku == 0);
+    using Cursor = GemvCursor<Source>;
+    auto seek = [&](Cursor &c) {  // to the first unit of the next stretch
+        if (!c.src.next(c.d, c.nb, c.ku, c.left, c.part, c.parts)) c.left = 0;
     };
-    auto advance = [&](GemvCursor &c) {
-        if (--c.left <= 0) {
-            seek(c);
-        } else if (++c.ku == c.d.k_units) {
-            c.ku = 0;
-            ++c.nb;
-        }
+    auto advance = [&](Cursor &c) {
+        if (--c.left <= 0) seek(c);
+        else ++c.ku;
     };
 
     constexpr int NG = kGemvCols / 16;  // 16 MFMA tiles per wave
@@ -181,7 +176,7 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
     // two units are kept in flight per wave (16 KB), in two register sets
     u32x4 stage_a[NLD], stage_b[NLD];
     u32x2 x_a, x_b;
-    auto gload = [&](const GemvCursor &c, u32x4(&stage)[NLD], u32x2 &xf) {
+    auto gload = [&](const Cursor &c, u32x4(&stage)[NLD], u32x2 &xf) {
         const GemvDesc &d = c.d;
         gptr<const T> W = as_global(static_cast<const T *>(d.w));
         gptr<const T> xsrc = as_global(static_cast<const T *>(d.x)) + (int64_t)xm * d.ldx + xk;
@@ -217,10 +212,10 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
         xf = xv;
     };
 
-    GemvCursor L, C;  // loads run two units ahead of the products
+    Cursor L(source);  // loads run two units ahead of the products
     seek(L);
     if (L.left <= 0) return;
-    C = L;
+    Cursor C = L;
     gload(L, stage_a, x_a);
     advance(L);
     if (L.left > 0) {
@@ -260,16 +255,16 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        const GemvDesc &d = C.d;
-        const int task = C.task, nb = C.nb;
-        const bool block_ends = (C.ku + 1 == d.k_units);
-        if (!block_ends && C.left > 1) return;
+        if (C.left > 1) return;
 
-        // ---- leaving column block nb: add the 8 waves' tiles through LDS ----------------
+        // ---- end of a stretch: add the 8 waves' tiles through LDS ------------------------
         // accumulator layout of 16x16x16: lane holds column (lane%16) = m and rows
         // 4*(lane/16) + r = n inside the tile
+        const GemvDesc &d = C.d;
+        const int nb = C.nb;
         gptr<T> Y = as_global(static_cast<T *>(d.y));
         s.sync();  // every wave is done with its staging window
+        C.src.fold_begins(tid);
         {
             lds_f32 *red = (lds_f32 *)wlds;
             const int m = lane & 15, nq = (lane >> 4) * 4;
@@ -310,8 +305,7 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
                 for (int e = 0; e < 4; ++e) p[e] = o[e];
             }
         };
-        const bool whole_block = C.from_zero && block_ends;
-        if (whole_block) {
+        if (C.parts == 1) {
             if (col < d.n) {
 #pragma unroll
                 for (int pass = 0; pass < 2; ++pass) {
@@ -320,7 +314,7 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
                 }
             }
         } else {
-            // K of this block is shared with other tasks: partial + arrival counter.
+            // K of this block is shared with other stretches: partial + arrival counter.
             // Partials travel as 16-byte buffer stores and loads with the agent-scope
             // bit (written through to memory, read past this XCD's L2), so no
             // cache-wide write-back or invalidate is needed: those are serialised
@@ -329,10 +323,7 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
             // before the workgroup barrier, the counter is bumped after it, and the
             // partials are read only after the counter has been seen full.
             constexpr int kAgentScope = 16;  // cache-policy bit sc1 of the buffer instructions
-            const int64_t U = (int64_t)d.n_blocks * d.k_units;
-            const int t_first = (int)gemv_task_of((int64_t)nb * d.k_units, U, d.num_tasks);
-            const int t_last = (int)gemv_task_of((int64_t)(nb + 1) * d.k_units - 1, U, d.num_tasks);
-            const int parts = t_last - t_first + 1;
+            const int parts = C.parts;
             const int part_bytes = d.m * kGemvCols * 4;
             float *Pb = d.partial + (int64_t)nb * d.max_parts * d.m * kGemvCols;
             const __amdgpu_buffer_rsrc_t rsrc =
@@ -342,7 +333,7 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
                 const int m = mrow + 8 * pass;
                 if (m < d.m)
                     __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, sums[pass]), rsrc,
-                                                           (task - t_first) * part_bytes + (m * kGemvCols + c4) * 4,
+                                                           C.part * part_bytes + (m * kGemvCols + c4) * 4,
                                                            0, kAgentScope);
             }
             drain_stores_then_barrier();
@@ -358,19 +349,21 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
                     for (int pass = 0; pass < 2; ++pass) {
                         const int m = mrow + 8 * pass;
                         if (m < d.m) {
-                            // four loads in flight per row, added in task order
+                            // eight loads in flight per row (the accumulator registers are
+                            // free here), added in the order of the parts
+                            constexpr int kInFlight = 8;
                             f32x4 v{0.f, 0.f, 0.f, 0.f};
-                            for (int q0 = 0; q0 < parts; q0 += 4) {
-                                u32x4 t[4];
+                            for (int q0 = 0; q0 < parts; q0 += kInFlight) {
+                                u32x4 t[kInFlight];
 #pragma unroll
-                                for (int i = 0; i < 4; ++i)
+                                for (int i = 0; i < kInFlight; ++i)
                                     t[i] = (q0 + i < parts)
                                                ? __builtin_amdgcn_raw_buffer_load_b128(
                                                      rsrc, (q0 + i) * part_bytes + (m * kGemvCols + c4) * 4, 0,
                                                      kAgentScope)
                                                : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
-                                for (int i = 0; i < 4; ++i)
+                                for (int i = 0; i < kInFlight; ++i)
                                     if (q0 + i < parts) v += __builtin_bit_cast(f32x4, t[i]);
                             }
                             store_y(m, v);
@@ -381,8 +374,8 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
                     __hip_atomic_store(d.counters + nb, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
-        s.sync();  // the windows (and the flag) are reused by the next segment
-        C.from_zero = block_ends;  // (a task that ends inside a block is followed by a new task)
+        C.src.fold_ends(tid);
+        s.sync();  // the windows (and the flag) are reused by the next stretch
     };
     for (;;) {
         consume(stage_a, x_a);
@@ -394,22 +387,41 @@ __device__ __forceinline__ void gemv_stream(const Slot &s, Source source) {
     }
 }
 
-// The tasks first, first + stride, ... < end of one skinny matmul, as one stream.
+// The stretches of the tasks first, first + stride, ... < end of one skinny matmul whose units are
+// dealt to d.num_tasks tasks in contiguous ranges (gemv_partition): a task's range, cut at the
+// column-block boundaries.
+struct GemvTaskSource {
+    const GemvDesc *d;
+    int t, stride, end;
+    int u = 0, u_end = 0;
+    __device__ __forceinline__ GemvTaskSource(const GemvDesc *desc, int first, int step, int last)
+        : d(desc), t(first - step), stride(step), end(last) {}
+    __device__ __forceinline__ bool next(GemvDesc &out, int &nb, int &ku, int &units, int &part, int &parts) {
+        const int64_t U = (int64_t)d->n_blocks * d->k_units;
+        while (u >= u_end) {
+            t += stride;
+            if (t >= end) return false;
+            u = (int)gemv_task_begin(t, U, d->num_tasks);
+            u_end = (int)gemv_task_begin(t + 1, U, d->num_tasks);
+        }
+        out = *d;
+        nb = u / d->k_units;
+        ku = u - nb * d->k_units;
+        units = min(u_end - u, d->k_units - ku);
+        const int t_first = (int)gemv_task_of((int64_t)nb * d->k_units, U, d->num_tasks);
+        const int t_last = (int)gemv_task_of((int64_t)(nb + 1) * d->k_units - 1, U, d->num_tasks);
+        part = t - t_first;
+        parts = t_last - t_first + 1;
+        u += units;
+        return true;
+    }
+    __device__ __forceinline__ void fold_begins(int) {}
+    __device__ __forceinline__ void fold_ends(int) {}
+};
+
 template <typename T>
 __device__ __forceinline__ void gemv_tasks(const GemvDesc &d, int first, int stride, int end, const Slot &s) {
-    const int64_t U = (int64_t)d.n_blocks * d.k_units;
-    gemv_stream<T>(s, [&](int i, GemvDesc &out, int &task, int &nb, int &ku, int &units) {
-        const int t = first + i * stride;
-        if (t >= end) return false;
-        // (every task has a unit: the partition never makes more tasks than units)
-        const int u_begin = (int)gemv_task_begin(t, U, d.num_tasks);
-        out = d;
-        task = t;
-        nb = u_begin / d.k_units;
-        ku = u_begin - nb * d.k_units;
-        units = (int)gemv_task_begin(t + 1, U, d.num_tasks) - u_begin;
-        return units > 0;
-    });
+    gemv_stream<T>(s, GemvTaskSource(&d, first, stride, end));
 }
 
 }  // namespace arkmi

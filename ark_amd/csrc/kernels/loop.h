@@ -62,17 +62,22 @@ struct DevTaskGroup {
     // As a producer: task index i completes row block signal_map[signal_begin + i] and adds one
     // to counter signal_base + that block; signal_begin < 0: the group signals nothing.
     int32_t signal_begin, signal_base;
-    // A group of skinny-matmul tasks runs from a table the host lays out, LoopProgram::gemv_seq:
-    // workgroup b's tasks of the group, in order, are the entries from seq_begin + b * seq_stride
-    // up to the first one with op < 0.  Groups that follow one another with nothing to wait for
-    // in between are streamed as one sequence by the loop kernel (the next matmul's weights are
-    // on their way while the current one adds up its tiles): chain = n > 1 on the first group
-    // of such a run (the groups gi .. gi + n - 1), whose chain_begin / chain_stride name the
-    // sequence of the whole run, and chain = -1 on the others, which the loop kernel skips.
-    // The one-op kernels run every group from its own table.
+    // A group of skinny-matmul tasks runs from tables the host lays out in LoopProgram::gemv_seq
+    // (stretches of units, GemvSeqEntry).  The one-op kernels run the group by itself: workgroup
+    // b's stretches are the entries from seq_begin + b * seq_stride up to the first one with
+    // op < 0.  The loop kernel streams runs of groups that follow one another with nothing to wait
+    // for in between as one sequence (the next matmul's weights are on their way while the current
+    // one adds up its tiles): chain = n > 1 on the first group of such a run (the groups gi ..
+    // gi + n - 1), -1 on the others, which the loop kernel skips, 0 on a group by itself.  The
+    // sequence of the run (or of the group by itself) is
+    //   claim < 0:  per workgroup, the entries from run_begin + b * run_stride as above;
+    //   claim >= 0: the run_stride entries from run_begin on, shared: workgroup b takes entries
+    //               b and b + grid and claims further ones from claim counter `claim` as it gets
+    //               free (LoopProgram::gemv_claims).
     int32_t chain;
     int32_t seq_begin, seq_stride;
-    int32_t chain_begin, chain_stride;
+    int32_t run_begin, run_stride;
+    int32_t claim;
 };
 
 // One producer a task group waits for.
@@ -140,7 +145,11 @@ struct LoopProgram {
     const int32_t *wait_spans;
     const int32_t *signal_map;
     unsigned int *dep_counters;
-    const GemvSeqEntry *gemv_seq;  // the task sequences of the skinny matmuls, null if there are none
+    const GemvSeqEntry *gemv_seq;  // the sequences of the skinny matmuls, null if there are none
+    // Claim counters of the skinny matmuls whose stretches are claimed at run time: two words per
+    // counter, kDepStride apart, used by alternating iterations (the one not in use is zeroed
+    // during the other's iteration; a grid barrier separates iterations).  Zero at every launch.
+    unsigned int *gemv_claims;
     int32_t num_steps;
     int32_t num_blocks;
     // what separates two iterations of the body inside one command:

@@ -403,47 +403,101 @@ ARKMI_BODY int gemm_f32_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, 
                           });
 }
 
-// This workgroup's skinny-matmul tasks from the sequence at `seq` (the host's table), one after
-// the other, with the loads running on across the boundaries between tasks and between matmuls.
-template <typename T>
-__device__ __forceinline__ void gemv_sequence(KArgs ka, const GemvSeqEntry *seq, const Slot &s) {
-    gemv_stream<T>(s, [&](int i, GemvDesc &out, int &task, int &nb, int &ku, int &units) {
-        const GemvSeqEntry e = load_const(seq + i);
+// Where the loop kernel's skinny-matmul stretches come from (the `Source` of gemv_stream).
+// This workgroup's row of one of the host's tables:
+struct GemvTableSource {
+    KArgs ka;
+    const GemvSeqEntry *entry;  // the next one
+    int tid;
+    __device__ __forceinline__ bool next(GemvDesc &d, int &nb, int &ku, int &units, int &part, int &parts) {
+        const GemvSeqEntry e = load_const(entry);
         if (e.op < 0) return false;
+        ++entry;
 #ifndef ARKMI_NO_TRACE
         TraceRecord *trace = KARG(prog.trace);
-        if (trace && e.trace_index >= 0 && s.tid == 0) {
+        if (trace && e.trace_index >= 0 && tid == 0) {
             TraceRecord rec{(int)blockIdx.x, 0, e.order};
             trace[e.trace_index] = rec;
         }
 #endif
-        out = load_const(&(KARG(prog.ops) + e.op)->gemv);
-        task = e.task;
-        nb = e.nb;
-        ku = e.ku;
-        units = e.units;
+        d = load_const(&(KARG(prog.ops) + e.op)->gemv);
+        nb = e.nb; ku = e.ku; units = e.units; part = e.part; parts = e.parts;
         return true;
-    });
-}
+    }
+    __device__ __forceinline__ void fold_begins(int) {}
+    __device__ __forceinline__ void fold_ends(int) {}
+};
+
+// A list of stretches shared by the grid: workgroup b streams entries b and b + grid, and while
+// it folds its k-th stretch it claims the one it will stream as its (k+2)-th from a counter, so a
+// workgroup that streams more slowly (its share of the HBM bandwidth varies) ends up with fewer.
+// Thread 0 claims; the claimed index reaches the other waves through a ring of four words in
+// the body's LDS control area, published by the barrier that ends the fold.  The load cursor,
+// two units ahead, reads position k when it leaves stretch k - 1, which is after the fold of
+// stretch k - 2 as long as every stretch has at least 3 units (the host checks).
+struct GemvClaimSource {
+    KArgs ka;
+    const GemvSeqEntry *entries;
+    int n;
+    unsigned *counter;  // of this iteration
+    unsigned *other;    // of the next one: zeroed meanwhile
+    lds_u32_ptr ring;
+    int k = 0;          // position of the next stretch in this workgroup's sequence
+    unsigned pending = 0;
+    __device__ __forceinline__ bool next(GemvDesc &d, int &nb, int &ku, int &units, int &part, int &parts) {
+        unsigned id;
+        if (k < 2) id = blockIdx.x + (unsigned)k * gridDim.x;
+        else id = __builtin_amdgcn_readfirstlane(ring[k & 3]);
+        ++k;
+        if (id >= (unsigned)n) return false;
+        const GemvSeqEntry e = load_const(entries + id);
+        d = load_const(&(KARG(prog.ops) + e.op)->gemv);
+        nb = e.nb; ku = e.ku; units = e.units; part = e.part; parts = e.parts;
+        return true;
+    }
+    // (called on the multiply cursor: k - 1 is the position of the stretch being folded)
+    __device__ __forceinline__ void fold_begins(int tid) {
+        if (tid == 0) {
+            pending = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, AGENT);
+            if (blockIdx.x == 0 && k == 1) __hip_atomic_store(other, 0u, __ATOMIC_RELAXED, AGENT);
+        }
+    }
+    __device__ __forceinline__ void fold_ends(int tid) {
+        if (tid == 0) ring[(k + 1) & 3] = pending + 2u * gridDim.x;
+    }
+};
 
 // (Skinny matmuls take no part in the dependency counters: the host keeps the barriers around
 // them, so there is nothing to wait for or to signal here.)
-ARKMI_BODY int gemv_body(KArgs ka_in, int gi_in, int t0, int tid, lds_ptr lds, unsigned epoch) {
+ARKMI_BODY int gemv_body(KArgs ka_in, int gi_in, int t0, int tid, lds_ptr lds, unsigned epoch_in) {
     const KArgs ka = uniform_kargs(ka_in);
     const Slot s = body_slot(tid, lds);
     const int gi = __builtin_amdgcn_readfirstlane(gi_in);
+    const unsigned epoch = __builtin_amdgcn_readfirstlane(epoch_in);
     const DevTaskGroup *g = KARG(prog.groups) + gi;
     // the loop kernel streams a run of groups from the first one; the one-op kernels (which name
     // their group in the kernel arguments) run every group by itself
-    const bool run = KARG(group) < 0 && load_const(&g->chain) > 1;
-    const int begin = run ? load_const(&g->chain_begin) : load_const(&g->seq_begin);
-    const int stride = run ? load_const(&g->chain_stride) : load_const(&g->seq_stride);
-    const GemvSeqEntry *seq = KARG(prog.gemv_seq) + begin + (size_t)blockIdx.x * stride;
+    const bool loop = KARG(group) < 0;
+    const int begin = loop ? load_const(&g->run_begin) : load_const(&g->seq_begin);
+    const int stride = loop ? load_const(&g->run_stride) : load_const(&g->seq_stride);
+    const int claim = loop ? load_const(&g->claim) : -1;
+    const GemvSeqEntry *seq = KARG(prog.gemv_seq) + begin;
+    // (one element type per sequence: checked on the host)
+    if (claim >= 0) {
+        if (stride <= 0) return kTasksDone;
+        unsigned *counters = KARG(prog.gemv_claims) + (size_t)claim * 2 * kDepStride;
+        GemvClaimSource src{ka, seq, stride, counters + (epoch & 1u) * kDepStride,
+                            counters + ((epoch + 1u) & 1u) * kDepStride, (lds_u32_ptr)(s.lds + 16)};
+        if (load_const(&(KARG(prog.ops) + load_const(&seq->op))->gemv.dtype) == 1) gemv_stream<f16>(s, src);
+        else gemv_stream<bf16>(s, src);
+        return kTasksDone;
+    }
+    seq += (size_t)blockIdx.x * stride;
     const int op = load_const(&seq->op);
     if (op >= 0) {
-        // (one element type per sequence: checked on the host)
-        if (load_const(&(KARG(prog.ops) + op)->gemv.dtype) == 1) gemv_sequence<f16>(ka, seq, s);
-        else gemv_sequence<bf16>(ka, seq, s);
+        GemvTableSource src{ka, seq, tid};
+        if (load_const(&(KARG(prog.ops) + op)->gemv.dtype) == 1) gemv_stream<f16>(s, src);
+        else gemv_stream<bf16>(s, src);
     }
     return kTasksDone;
 }
@@ -587,9 +641,9 @@ __device__ __forceinline__ bool run_group(KArgs ka, const LoopProgram &P, int gi
         if (KARG(group) < 0) {
             // a skinny matmul that the first group of its run has already streamed
             if (g.chain < 0) return true;
-            // the first group of a run: the host's table says what this workgroup does for the
-            // run, whether or not it has a task of the first matmul
-            if (g.chain > 1) {
+            // the first group of a run, or stretches claimed at run time: the host's tables say
+            // what this workgroup does, whether or not it has a task of the (first) matmul
+            if (g.chain > 1 || g.claim >= 0) {
                 const Slot s0 = body_slot(threadIdx.x, (lds_ptr)g_loop_lds + kLdsReserved);
                 return run_long_tasks<FAM, DEV_GEMV>(ka, gi, s0, epoch);
             }

@@ -27,7 +27,7 @@ class ExecInfo(ctypes.Structure):
                 ("destroyed", ctypes.c_int), ("loop_mode", ctypes.c_int),
                 ("iterations_done", ctypes.c_int), ("barriers_local", ctypes.c_int),
                 ("iteration_sync", ctypes.c_int), ("barriers_counted", ctypes.c_int),
-                ("gemv_chains", ctypes.c_int)]
+                ("gemv_chains", ctypes.c_int), ("gemv_claimed", ctypes.c_int)]
 
 
 def _i64(v):

@@ -263,6 +263,7 @@ typedef struct arkmi_exec_info_t {
     int iteration_sync;   /* between iterations of one run(n): 2 grid barrier, 1 workgroup-local sync, 0 nothing */
     int barriers_counted; /* grid barriers replaced by waits on per-row-block dependency counters */
     int gemv_chains;      /* runs of consecutive skinny matmuls that the loop kernel streams as one sequence */
+    int gemv_claimed;     /* skinny matmuls (or runs) whose stretches the workgroups claim at run time */
 } arkmi_exec_info_t;
 
 int arkmi_exec_create(int device_id, void *stream, const char *name,

@@ -146,22 +146,25 @@ def test_analysis_rejects_what_compile_rejects():
 def test_consecutive_skinny_matmuls_form_one_stream():
     """Skinny matmuls that follow one another with no barrier or sync between them are marked as one
     run (the first group carries the length, the others -1); anything in between, a dependency, or
-    an op fused into the task breaks the run."""
+    another element type breaks the run.  A run (or a matmul by itself) whose column blocks all have
+    at least three units is cut into stretches that the workgroups claim at run time."""
     m = Model()
     for k, n in [(4096, 12288), (4096, 4096), (4096, 22016), (11008, 4096)]:
         m.matmul(m.tensor([1, k], "bf16"), m.tensor([k, n], "bf16"))
-    a = plan_analysis(_plan(m), 0)
-    assert a["GemvChains"] == 1
+    plan = _plan(m)
+    a = plan_analysis(plan, 0)
+    assert a["GemvChains"] == 1 and a["GemvClaimed"] == 1
     assert [s["Kind"] for s in a["Steps"]] == ["Tasks"] * 4
-    assert [s["Chain"] for s in a["Steps"]] == [4, -1, -1, -1]
+    assert [(s["Chain"], s["Claimed"]) for s in a["Steps"]] == [(4, True), (-1, False), (-1, False), (-1, False)]
 
-    # y2 depends on y1: the barrier between them stays and nothing is chained
+    # y2 depends on y1: the barrier between them stays, nothing is chained, each claims by itself
     m = Model()
     y1 = m.matmul(m.tensor([1, 4096], "bf16"), m.tensor([4096, 4096], "bf16"))
     m.matmul(y1, m.tensor([4096, 4096], "bf16"))
     a = plan_analysis(_plan(m), 0)
     assert a["GemvChains"] == 0 and [s["Kind"] for s in a["Steps"]] == ["Tasks", "Barrier", "Tasks"]
-    assert [s["Chain"] for s in _tasks_steps(a)] == [0, 0]
+    assert [(s["Chain"], s["Claimed"]) for s in _tasks_steps(a)] == [(0, True), (0, True)]
+    assert a["GemvClaimed"] == 2 and a["IterationSync"] == 2
 
     # two runs separated by an elementwise op of its own
     m = Model()
@@ -170,8 +173,10 @@ def test_consecutive_skinny_matmuls_form_one_stream():
     m.relu(m.tensor([64, 64], "fp16"))
     for _ in range(3):
         m.matmul(m.tensor([2, 1024], "fp16"), m.tensor([1024, 512], "fp16"))
-    # a different element type does not join the run before it
-    m.matmul(m.tensor([2, 1024], "bf16"), m.tensor([1024, 512], "bf16"))
+    # a different element type does not join the run before it; K = 256 is two units: too few to
+    # cut into claimable stretches
+    m.matmul(m.tensor([2, 256], "bf16"), m.tensor([256, 512], "bf16"))
     a = plan_analysis(_plan(m), 0)
-    assert a["GemvChains"] == 2
-    assert [s["Chain"] for s in _tasks_steps(a)] == [2, -1, 0, 3, -1, -1, 0]
+    assert a["GemvChains"] == 2 and a["GemvClaimed"] == 2
+    assert [(s["Chain"], s["Claimed"]) for s in _tasks_steps(a)] == [
+        (2, True), (-1, False), (0, False), (3, True), (-1, False), (-1, False), (0, False)]

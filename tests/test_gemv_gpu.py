@@ -162,7 +162,7 @@ def test_decode_step_four_projections_in_one_plan(oracle, batch):
         vals[tw] = make(oracle, (k, n), dtype, seed=50 + i, dist="normal", scale=0.02)
         xs.append(tx); ws.append(tw); ys.append(mod.matmul(tx, tw))
     ex = Executor(mod.plan(device_id=0)).compile()
-    assert ex.info()["kernel_families"] == 8 and ex.info()["gemv_chains"] == 1
+    assert ex.info()["kernel_families"] == 8 and ex.info()["gemv_chains"] == 1 and ex.info()["gemv_claimed"] == 1
     for t, a in vals.items():
         ex.tensor_write(t, a)
     ex.launch()
@@ -177,14 +177,21 @@ def test_decode_step_four_projections_in_one_plan(oracle, batch):
 
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
-def test_consecutive_skinny_matmuls_run_as_one_stream(oracle, dtype, monkeypatch):
+@pytest.mark.parametrize("claimed", [False, True])
+def test_consecutive_skinny_matmuls_run_as_one_stream(oracle, dtype, claimed, monkeypatch):
     """Independent skinny matmuls that follow one another are streamed as one sequence by the loop
-    kernel (the next one's weights are loaded while the current one adds up its tiles).  Shapes with
-    ragged K and N, different row counts, few tasks (most workgroups have nothing to do for that
-    matmul) and many: every output against the oracle, and bit for bit against the same plan with
-    the matmuls run one by one (ARKMI_GEMV_CHAIN=0) and as one kernel per op."""
+    kernel (the next one's weights are loaded while the current one adds up its tiles), and when all
+    of them are deep enough the workgroups claim their stretches at run time instead of getting fixed
+    shares.  Shapes with ragged K and N, different row counts, few stretches (most workgroups have
+    nothing to do for that matmul) and many: every output against the oracle, and bit for bit
+    against the same plan with fixed shares (ARKMI_GEMV_CLAIM=0), with the matmuls run one by one
+    (ARKMI_GEMV_CHAIN=0) and as one kernel per op: the partial sums are per stretch and added in a
+    fixed order, whoever streams them."""
     from ark_amd import Model, Executor
-    shapes = [(1, 2048, 1536), (3, 296, 264), (8, 4096, 512), (16, 1024, 8), (2, 16, 4096), (1, 11008, 1024)]
+    if claimed:
+        shapes = [(1, 2048, 1536), (3, 424, 264), (8, 4096, 512), (16, 1024, 8), (2, 384, 4096), (1, 11008, 1024)]
+    else:  # a matmul of one or two units keeps the run on fixed shares
+        shapes = [(1, 2048, 1536), (3, 296, 264), (8, 4096, 512), (16, 1024, 8), (2, 16, 4096), (1, 11008, 1024)]
     mod = Model()
     vals, ys = {}, []
     for i, (m, k, n) in enumerate(shapes):
@@ -194,7 +201,7 @@ def test_consecutive_skinny_matmuls_run_as_one_stream(oracle, dtype, monkeypatch
         ys.append((mod.matmul(tx, tw), tx, tw, k))
     plan = mod.plan(device_id=0)
 
-    def run(separate=False):
+    def run(separate=False, iters=3):
         ex = Executor(plan, device_id=0, loop_mode=not separate).compile()
         info = ex.info()
         for t, a in vals.items():
@@ -204,20 +211,42 @@ def test_consecutive_skinny_matmuls_run_as_one_stream(oracle, dtype, monkeypatch
             torch.cuda.synchronize()
         else:
             ex.launch()
-            ex.run(3)
+            ex.run(iters)
+            ex.wait()
+            ex.run(2)  # (a second command: the claim counters alternate by iteration across commands)
             ex.wait()
         got = [ex.tensor_read(y) for y, _, _, _ in ys]
         if not separate:
             ex.stop()
         return got, info
 
-    chained, info = run()
-    assert info["kernel_families"] == 8 and info["gemv_chains"] == 1
-    for g, (_, tx, tw, k) in zip(chained, ys):
+    first, info = run()
+    assert info["kernel_families"] == 8 and info["gemv_chains"] == 1 and info["gemv_claimed"] == int(claimed)
+    for g, (_, tx, tw, k) in zip(first, ys):
         _check(oracle, oracle.matmul(vals[tx], vals[tw], dtype), g, dtype, 4.0 * 0.25, k)
-    one_kernel_per_op, _ = run(separate=True)
+    # who streams what does not matter: another run of the same plan gives the same bits
+    again, _ = run(iters=4)
+    for a, b in zip(first, again):
+        assert np.array_equal(a, b)
+    # fixed shares: the plan's tasks, the same in a run, one by one and as one kernel per op
+    monkeypatch.setenv("ARKMI_GEMV_CLAIM", "0")
+    fixed, info = run()
+    assert info["gemv_chains"] == 1 and info["gemv_claimed"] == 0
     monkeypatch.setenv("ARKMI_GEMV_CHAIN", "0")
     one_by_one, info = run()
-    assert info["gemv_chains"] == 0
-    for a, b, c in zip(chained, one_by_one, one_kernel_per_op):
+    assert info["gemv_chains"] == 0 and info["gemv_claimed"] == 0
+    one_kernel_per_op, _ = run(separate=True)
+    for a, b, c in zip(fixed, one_by_one, one_kernel_per_op):
         assert np.array_equal(a, b) and np.array_equal(a, c)
+    for g, (_, tx, tw, k) in zip(fixed, ys):
+        _check(oracle, oracle.matmul(vals[tx], vals[tw], dtype), g, dtype, 4.0 * 0.25, k)
+    if not claimed:
+        for a, b in zip(first, fixed):
+            assert np.array_equal(a, b)
+    # every matmul by itself, its stretches claimed where it is deep enough (cut differently from
+    # the run: other partial sums, same tolerance)
+    monkeypatch.delenv("ARKMI_GEMV_CLAIM")
+    alone, info = run()
+    assert info["gemv_chains"] == 0 and info["gemv_claimed"] == (6 if claimed else 5)
+    for g, (_, tx, tw, k) in zip(alone, ys):
+        _check(oracle, oracle.matmul(vals[tx], vals[tw], dtype), g, dtype, 4.0 * 0.25, k)
