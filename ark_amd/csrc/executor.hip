@@ -1125,6 +1125,7 @@ struct Executor {
     GemvSeqEntry *d_gemv_seq = nullptr;
     unsigned int *d_gemv_claims = nullptr;
     size_t gemv_claim_bytes = 0;
+    int barriers_widened = 0;               // barriers over part of the grid made full-grid for claimed stretches
     int gemv_claimed = 0;                   // skinny matmuls (or runs of them) whose stretches are claimed at run time
     std::vector<GemvSeqEntry> h_gemv_seq;  // the skinny matmuls' task sequences, per workgroup
     std::vector<int> group_sched_step;      // schedule step of every task group
@@ -1625,6 +1626,7 @@ struct Executor {
         //    (ARKMI_GEMV_CLAIM=0: the tasks' fixed shares).
         gemv_chains = 0;
         gemv_claimed = 0;
+        barriers_widened = 0;
         h_gemv_seq.clear();
         {
             const char *chain_env = getenv("ARKMI_GEMV_CHAIN"), *claim_env = getenv("ARKMI_GEMV_CLAIM");
@@ -1684,14 +1686,24 @@ struct Executor {
                 }
             };
             // claimed at run time: possible when every column block has the 3 units a stretch needs
-            // (the claim protocol's look-ahead) and the plan's barriers span the grid
-            // (every workgroup of the grid then streams for the matmul, whatever processors the
-            // plan names for it; a barrier over part of the grid would not wait for all of them)
-            bool whole_grid_barriers = true;
-            for (const DevStep &st : steps)  // (the barriers that are left)
-                if (st.kind == STEP_BARRIER && st.count != grid) whole_grid_barriers = false;
+            // (the claim protocol's look-ahead).  Every workgroup of the grid then streams for the
+            // matmul, whatever processors the plan names for it, and a barrier over part of the grid
+            // would not wait for all of them: a plan that has such a matmul gets its remaining
+            // barriers over part of the grid widened to the whole grid (a stronger order, reached
+            // by every workgroup in the same place).
+            bool any_claimable = false;
+            for (const DevTaskGroup &g : h_groups)
+                if (claim_on && is_gemv(g) && g.n_waits == 0 && g.signal_begin < 0 &&
+                    ops[(size_t)g.op_begin].gemv.k_units >= kGemvMinStretch)
+                    any_claimable = true;
+            if (any_claimable)
+                for (DevStep &st : steps)
+                    if (st.kind == STEP_BARRIER && st.count != grid) {
+                        st.b = 0; st.e = grid; st.s = 1; st.count = grid;
+                        ++barriers_widened;
+                    }
             auto claimable = [&](size_t first, size_t n) {
-                if (!claim_on || !whole_grid_barriers) return false;
+                if (!claim_on) return false;
                 for (size_t gi = first; gi < first + n; ++gi)
                     if (ops[(size_t)h_groups[gi].op_begin].gemv.k_units < kGemvMinStretch) return false;
                 return true;
@@ -2334,6 +2346,7 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
         out["BarriersCounted"] = (long long)ex.barriers_counted;
         out["GemvChains"] = (long long)ex.gemv_chains;
         out["GemvClaimed"] = (long long)ex.gemv_claimed;
+        out["BarriersWidened"] = (long long)ex.barriers_widened;
         out["IterationSync"] = (long long)ex.iteration_sync;
         out["NumCounters"] = (long long)ex.dry_counters;
         Json steps = Json::array();

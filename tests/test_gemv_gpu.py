@@ -250,3 +250,58 @@ def test_consecutive_skinny_matmuls_run_as_one_stream(oracle, dtype, claimed, mo
     assert info["gemv_chains"] == 0 and info["gemv_claimed"] == (6 if claimed else 5)
     for g, (_, tx, tw, k) in zip(alone, ys):
         _check(oracle, oracle.matmul(vals[tx], vals[tw], dtype), g, dtype, 4.0 * 0.25, k)
+
+
+@pytest.mark.parametrize("num_processors", [256, 40])
+def test_dependent_skinny_matmuls_claim_their_stretches(oracle, num_processors, monkeypatch):
+    """y = ((x W1) W2) W3 with 2 rows: every matmul waits for the one before it (the grid barriers
+    stay), and each is cut into stretches that the workgroups claim at run time, with their two claim
+    counters alternating over the iterations of several commands.  On the full grid and on 40
+    processors (more stretches than twice the workgroups: most are claimed, few are the fixed first
+    two).  Against the oracle and the plan's fixed shares (three bf16 roundings deep, a last-bit
+    difference of an intermediate value moves a result by an ulp or two: judged by the largest
+    difference against the largest value, 1e-2), and bit for bit against a second run."""
+    from ark_amd import Model, Executor
+    dtype = "bf16"
+    dims = [(2048, 3072), (3072, 1024), (1024, 2048)]
+    mod = Model()
+    tx = mod.tensor([2, dims[0][0]], dtype)
+    vals = {tx: make(oracle, (2, dims[0][0]), dtype, seed=90, dist="normal")}
+    ws, y = [], tx
+    for i, (k, n) in enumerate(dims):
+        tw = mod.tensor([k, n], dtype)
+        vals[tw] = make(oracle, (k, n), dtype, seed=91 + i, dist="normal", scale=0.03)
+        ws.append(tw)
+        y = mod.matmul(y, tw)
+    plan = mod.plan(arch="ROCM_950", num_processors=num_processors)
+
+    def run(commands):
+        ex = Executor(plan, device_id=0).compile()
+        info = ex.info()
+        for t, a in vals.items():
+            ex.tensor_write(t, a)
+        ex.launch()
+        for n in commands:
+            ex.run(n)
+            ex.wait()
+        got = ex.tensor_read(y)
+        ex.stop()
+        return got, info
+
+    got, info = run([1, 2, 3])
+    assert info["gemv_chains"] == 0 and info["gemv_claimed"] == 3 and info["iteration_sync"] == 2
+    assert info["num_processors"] <= num_processors  # (a plan names the processors it uses)
+    ref = vals[tx]
+    for tw in ws:
+        ref = oracle.matmul(ref, vals[tw], dtype)
+    ref32 = oracle.to_f32(ref, dtype)
+
+    def close(a):
+        return float(np.abs(oracle.to_f32(a, dtype) - ref32).max()) <= 1e-2 * float(np.abs(ref32).max())
+    assert close(got)
+    again, _ = run([4])
+    assert np.array_equal(got, again)
+    monkeypatch.setenv("ARKMI_GEMV_CLAIM", "0")
+    fixed, info = run([2])
+    assert info["gemv_claimed"] == 0
+    assert close(fixed)
