@@ -663,8 +663,13 @@ DevOp lower_op(const Json &op_json, const Lowering &L, int slot_warps, int block
         }
         if (w.dt_in != w.dt_out && e.op != EW_CAST)
             ARK_ERR(PlanError, "op ", type, ": input and output types differ");
-        if ((w.dt_in == 3 || w.dt_out == 3) && e.op != EW_CAST && e.op != EW_COPY)
-            ARK_ERR(UnsupportedError, "op ", type, " is not implemented for INT32");
+        {
+            const bool int_ok = e.op == EW_CAST || e.op == EW_COPY || e.op == EW_ADD || e.op == EW_SUB ||
+                                e.op == EW_MUL || e.op == EW_DIV || e.op == EW_SCALAR_ASSIGN ||
+                                e.op == EW_SCALAR_ADD || e.op == EW_SCALAR_MUL;
+            if ((w.dt_in == 3 || w.dt_out == 3) && !int_ok)
+                ARK_ERR(UnsupportedError, "op ", type, " is not implemented for INT32");
+        }
         if (e.op == EW_ROPE && (out.shape[3] % 2) != 0)
             ARK_ERR(PlanError, "Rope needs an even innermost dimension");
         w.op = e.op;

@@ -24,7 +24,13 @@ enum EwOp : int32_t {
     EW_EXP, EW_GELU, EW_RELU, EW_RSQRT, EW_SIGMOID, EW_SQRT,  // unary
     EW_COPY, EW_CAST,
     EW_SCALAR_ASSIGN, EW_SCALAR_ADD, EW_SCALAR_MUL,
+    // INT32 tensors: the same ops on the bits (the values travel through the float registers of
+    // the common paths unconverted; the host selects these for dt_in == dt_out == int32)
+    EW_IADD, EW_ISUB, EW_IMUL, EW_IDIV, EW_ISCALAR_ASSIGN, EW_ISCALAR_ADD, EW_ISCALAR_MUL,
 };
+
+constexpr bool ew_is_binary(int op) { return op <= EW_ROPE || (op >= EW_IADD && op <= EW_IDIV); }
+constexpr bool ew_has_no_input(int op) { return op == EW_SCALAR_ASSIGN || op == EW_ISCALAR_ASSIGN; }
 
 struct EwTensor {
     void *ptr;
@@ -139,6 +145,25 @@ __device__ __forceinline__ void ew_compute(const float (&a)[kEwGroup], const flo
             case EW_SCALAR_ASSIGN: r = param; break;
             case EW_SCALAR_ADD: r = x + param; break;
             case EW_SCALAR_MUL: r = x * param; break;
+            // INT32: two's-complement wrap-around for + - *, C's truncating division (x / 0 and
+            // INT_MIN / -1 give 0 here), the scalar converted like a C cast
+            case EW_IADD: case EW_ISUB: case EW_IMUL: case EW_IDIV:
+            case EW_ISCALAR_ASSIGN: case EW_ISCALAR_ADD: case EW_ISCALAR_MUL: {
+                const bool scalar = OP >= EW_ISCALAR_ASSIGN;
+                const uint32_t ua = __builtin_bit_cast(uint32_t, x);
+                const uint32_t ub = scalar ? (uint32_t)(int32_t)param : __builtin_bit_cast(uint32_t, b[j]);
+                uint32_t ur;
+                if (OP == EW_IADD || OP == EW_ISCALAR_ADD) ur = ua + ub;
+                else if (OP == EW_ISUB) ur = ua - ub;
+                else if (OP == EW_IMUL || OP == EW_ISCALAR_MUL) ur = ua * ub;
+                else if (OP == EW_ISCALAR_ASSIGN) ur = ub;
+                else {
+                    const int32_t ia = (int32_t)ua, ib = (int32_t)ub;
+                    ur = (ib == 0 || (ia == INT32_MIN && ib == -1)) ? 0u : (uint32_t)(ia / ib);
+                }
+                r = __builtin_bit_cast(float, ur);
+                break;
+            }
             default: r = x; break;  // copy, cast
         }
         y[j] = r;
@@ -155,8 +180,8 @@ __device__ __forceinline__ void ew_compute(const float (&a)[kEwGroup], const flo
 template <typename TI, typename TO, int OP, bool PERIODIC = false>
 __device__ __forceinline__ void ewise_fast(const EwiseDesc &d, int n, int c, int h0, int h1, int w0, int w1,
                                            const Slot &s) {
-    constexpr bool BINARY = (OP <= EW_ROPE);
-    constexpr bool NO_INPUT = (OP == EW_SCALAR_ASSIGN);
+    constexpr bool BINARY = ew_is_binary(OP);
+    constexpr bool NO_INPUT = ew_has_no_input(OP);
     constexpr int U = kEwUnroll;
     using rawi = uint32_t __attribute__((ext_vector_type(sizeof(TI) * kEwGroup / 4)));
     using rawo = uint32_t __attribute__((ext_vector_type(sizeof(TO) * kEwGroup / 4)));
@@ -274,8 +299,8 @@ __device__ __forceinline__ void ewise_fast(const EwiseDesc &d, int n, int c, int
 
 template <typename TI, typename TO, int OP>
 __device__ __forceinline__ void ewise_task(const EwiseDesc &d, int task, const Slot &s) {
-    constexpr bool BINARY = (OP <= EW_ROPE);
-    constexpr bool NO_INPUT = (OP == EW_SCALAR_ASSIGN);
+    constexpr bool BINARY = ew_is_binary(OP);
+    constexpr bool NO_INPUT = ew_has_no_input(OP);
     const int tw_i = task % d.tiles_w;
     int t = task / d.tiles_w;
     const int th_i = t % d.tiles_h;
@@ -421,9 +446,20 @@ __device__ __forceinline__ void ewise_dispatch(const EwiseDesc &d, int task, con
         case 0: ewise_same_type<float>(d, task, s); break;
         case 1: ewise_same_type<f16>(d, task, s); break;
         case 2: ewise_same_type<bf16>(d, task, s); break;
-        // a same-type int32 copy moves the bits untouched (through float it would
-        // round values above 2^24)
-        default: ewise_task<float, float, EW_COPY>(d, task, s); break;
+        // int32: the bits travel untouched as 4-byte words (through a float conversion values
+        // above 2^24 would round); the arithmetic ops work on the bits
+        default:
+            switch (d.op) {
+                case EW_ADD: ewise_task<float, float, EW_IADD>(d, task, s); break;
+                case EW_SUB: ewise_task<float, float, EW_ISUB>(d, task, s); break;
+                case EW_MUL: ewise_task<float, float, EW_IMUL>(d, task, s); break;
+                case EW_DIV: ewise_task<float, float, EW_IDIV>(d, task, s); break;
+                case EW_SCALAR_ASSIGN: ewise_task<float, float, EW_ISCALAR_ASSIGN>(d, task, s); break;
+                case EW_SCALAR_ADD: ewise_task<float, float, EW_ISCALAR_ADD>(d, task, s); break;
+                case EW_SCALAR_MUL: ewise_task<float, float, EW_ISCALAR_MUL>(d, task, s); break;
+                default: ewise_task<float, float, EW_COPY>(d, task, s); break;
+            }
+            break;
     }
 }
 

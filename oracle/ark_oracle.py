@@ -207,7 +207,30 @@ def unary(x, kind, dtype):
     return out
 
 
+def _int32_op(a, b, kind):
+    """INT32 arithmetic as C computes it on two's-complement words: + - * wrap around, / truncates
+    toward zero (the reference's functors are `a + b` ... `a / b` on the element type,
+    ark/include/kernels/common/type_intrinsics.h:174-252; a scalar op casts its float value to the
+    element type first, ark/include/kernels/scalar.h:13-41).  x / 0 and INT_MIN / -1, undefined in C, are 0 here."""
+    a64, b64 = np.asarray(a, np.int32).astype(np.int64), np.asarray(b, np.int32).astype(np.int64)
+    if kind == "add":
+        r = a64 + b64
+    elif kind == "sub":
+        r = a64 - b64
+    elif kind == "mul":
+        r = a64 * b64  # |product| < 2^62: exact in int64
+    else:
+        bad = (b64 == 0) | ((a64 == -2 ** 31) & (b64 == -1))
+        safe = np.where(bad, 1, b64)
+        q = np.abs(a64) // np.abs(safe)
+        r = np.where(bad, 0, np.where((a64 < 0) != (safe < 0), -q, q))
+    return (r & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
+
+
 def binary(a, b, kind, dtype):
+    if dtype == "int32":
+        a, b = np.broadcast_arrays(np.asarray(a, np.int32), np.asarray(b, np.int32))
+        return _int32_op(a, b, kind)
     a = _c(a, dtype)
     b = _c(b, dtype)
     oshape = np.broadcast_shapes(a.shape, b.shape)
@@ -222,6 +245,10 @@ def binary(a, b, kind, dtype):
 
 
 def scalar(x, factor, kind, dtype):
+    if dtype == "int32":  # the factor is converted like a C cast (toward zero)
+        x = np.asarray(x, np.int32)
+        f = np.full(x.shape, int(np.float32(factor)), np.int32)
+        return f if kind == "assign" else _int32_op(x, f, kind)
     x = _c(x, dtype)
     out = np.empty_like(x)
     lib().orc_scalar(_p(x), _p(out), ctypes.c_int64(x.size),

@@ -326,3 +326,32 @@ def test_embedding_oracle_by_brute_force(oracle):
     flat = np.where(idx.reshape(-1) < 0, idx.reshape(-1) + 7, idx.reshape(-1))
     onehot[np.arange(6), flat] = 1.0
     assert np.array_equal(got.reshape(6, 5), onehot @ table)
+
+
+def test_int32_arithmetic_by_python_integers(oracle):
+    """INT32 add/sub/mul/div of the oracle against Python's unbounded integers reduced to 32-bit
+    two's complement, on values that overflow, and C's truncation toward zero for the quotient."""
+    rng = np.random.default_rng(3)
+    a = rng.integers(-2 ** 31, 2 ** 31, 4096, dtype=np.int64).astype(np.int32)
+    b = rng.integers(-2 ** 31, 2 ** 31, 4096, dtype=np.int64).astype(np.int32)
+    b[:64] = rng.integers(-9, 10, 64)  # small divisors, zeros among them
+    a[64:72] = -2 ** 31
+    b[64:72] = -1
+
+    def wrap(v):
+        v &= 0xFFFFFFFF
+        return v - (1 << 32) if v >= 1 << 31 else v
+
+    def cdiv(x, y):
+        if y == 0 or (x == -2 ** 31 and y == -1):
+            return 0
+        q = abs(x) // abs(y)
+        return -q if (x < 0) != (y < 0) else q
+    for kind, f in (("add", lambda x, y: wrap(x + y)), ("sub", lambda x, y: wrap(x - y)),
+                    ("mul", lambda x, y: wrap(x * y)), ("div", cdiv)):
+        want = np.array([f(int(x), int(y)) for x, y in zip(a, b)], np.int64).astype(np.int32)
+        assert np.array_equal(oracle.binary(a, b, kind, "int32"), want), kind
+    assert list(oracle.binary(np.array([7, -7, 7, -7], np.int32), np.array([2, 2, -2, -2], np.int32), "div", "int32")) == [3, -3, -3, 3]
+    assert list(oracle.scalar(np.array([5, -5], np.int32), 2.9, "mul", "int32")) == [10, -10]
+    assert list(oracle.scalar(np.array([5, -5], np.int32), -2.9, "add", "int32")) == [3, -7]
+    assert list(oracle.scalar(np.array([5, -5], np.int32), 7.0, "assign", "int32")) == [7, 7]
