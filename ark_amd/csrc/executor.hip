@@ -1124,18 +1124,21 @@ struct Executor {
     std::vector<DevStep> dry_steps;
     std::vector<DevWait> dry_waits;
     std::vector<int32_t> dry_spans, dry_signal;
+    std::vector<DevOp> dry_ops;
     size_t dry_counters = 0;
     DevWait *d_waits = nullptr;
     int32_t *d_spans = nullptr, *d_signal = nullptr;
     GemvSeqEntry *d_gemv_seq = nullptr;
     unsigned int *d_gemv_claims = nullptr;
     size_t gemv_claim_bytes = 0;
+    int gemm_xcd_ordered = 0;               // matmuls whose tiles run in the XCD-aware order
     int barriers_widened = 0;               // barriers over part of the grid made full-grid for claimed stretches
     int gemv_claimed = 0;                   // skinny matmuls (or runs of them) whose stretches are claimed at run time
     std::vector<GemvSeqEntry> h_gemv_seq;  // the skinny matmuls' task sequences, per workgroup
     std::vector<int> group_sched_step;      // schedule step of every task group
     unsigned int *d_dep_counters = nullptr;
     size_t dep_counter_bytes = 0;
+    bool iteration_local_across_groups = false;  // the local sync between iterations pairs two different groups
     int iteration_sync = 2;       // between iterations of one command: 2 grid barrier, 1 local sync, 0 nothing
     int families = 0;             // OpFamily bits of the compiled ops
     int kernel_families = 0;      // the loop-kernel variant in use
@@ -1559,6 +1562,7 @@ struct Executor {
         // workgroups, task by task, so its own tensors are a local matter unless an
         // op keeps partial results in scratch memory that other workgroups finish.
         iteration_sync = 2;
+        iteration_local_across_groups = false;
         if (elide) {
             bool whole_grid_only = true;
             int first_full = -1, last_full = -1;
@@ -1598,8 +1602,10 @@ struct Executor {
                             local = false;
                         else if (x.step == y.step)
                             local = !x.panel_read && !y.panel_read && x.view == y.view && x.begin == y.begin;
-                        else
+                        else {
                             local = local_pair(x, y);
+                            if (local) iteration_local_across_groups = true;
+                        }
                         if (!local) all_local = false;
                     }
                 iteration_sync = !any ? 0 : all_local ? 1 : 2;
@@ -1615,6 +1621,48 @@ struct Executor {
         // the counters count per iteration, and a reader relies on the caches having been
         // invalidated since the previous one
         if (barriers_counted > 0) iteration_sync = 2;
+
+        // ---- matmul tiles in an XCD-aware order ---------------------------------------------------
+        // Workgroups go to the eight XCDs round robin, and each XCD has an L2 of its own: with the
+        // tiles in row-major task order, the tiles an XCD works on at a time lie strewn over the
+        // output, and its L2 fetches nearly all of A (C1: 345 MB fetched for 67 MB of operands).
+        // Where task t runs on workgroup t mod R, the matmul's tile index is permuted so that they
+        // form a compact block (gemm_tile).  The tasks stay on their workgroups; the tile a task
+        // computes changes, and the ops fused behind the matmul follow it.  ARKMI_GEMM_XCD=0: off.
+        gemm_xcd_ordered = 0;
+        {
+            const char *xe = getenv("ARKMI_GEMM_XCD");
+            // (a workgroup-local sync in place of a barrier rests on task t of both ops running on
+            // the same workgroup for the same tile: plans that have one, inside the body or between
+            // two groups across the iteration boundary, keep the plain order; a group that meets
+            // only itself across iterations still computes the same tile on the same workgroup)
+            const bool on = !(xe && atoi(xe) == 0) && !trace_enabled && barriers_local == 0 &&
+                            !(iteration_sync == 1 && iteration_local_across_groups);
+            for (DevTaskGroup &g : h_groups) {
+                DevOp &op0 = ops[(size_t)g.op_begin];
+                if (!on || op0.kind != DEV_GEMM || op0.gemm.dtype == 0) continue;
+                GemmDesc &d = op0.gemm;
+                if (d.batch_total != 1 || g.n_waits > 0 || g.signal_begin >= 0) continue;  // (waits go by task index)
+                if (g.proc_b != 0 || g.proc_s != 1 || g.proc_cur != 0 || g.task_b != 0 || g.task_s != 1 || g.gran != 1)
+                    continue;
+                const int n_procs = g.proc_e, tiles = d.tiles_m * d.tiles_n;
+                const int round = std::min(tiles, n_procs);  // tiles in flight at once
+                if (n_procs % 8 != 0 || tiles % 8 != 0 || round % 8 != 0 || round < 16) continue;
+                if (g.task_e != tiles * (d.split_k == 2 ? 2 : 1)) continue;
+                const int per = round / 8, cols_cost = op0.gemm_tile_n * (d.b2 ? 2 : 1);
+                int best = 0;
+                long best_cost = 0;
+                for (int bm = 1; bm <= per; bm *= 2) {
+                    if (d.tiles_m % bm != 0 || per % bm != 0) continue;
+                    const long cost = (long)bm * op0.gemm_tile_m + (long)(per / bm) * cols_cost;
+                    if (best == 0 || cost < best_cost) { best = bm; best_cost = cost; }
+                }
+                if (best == 0) continue;
+                d.xcd_round = round;
+                d.xcd_band = best;
+                ++gemm_xcd_ordered;
+            }
+        }
 
         // ---- skinny matmuls: stretches, who streams which, runs of matmuls as one stream ----------
         // A workgroup streams stretches of consecutive units of one column block and folds at the
@@ -1785,6 +1833,7 @@ struct Executor {
         if (dry) {
             (void)loop_kernel_select(families, &kernel_families);
             dry_steps = steps;
+            dry_ops = ops;
             dry_waits = h_waits;
             dry_spans = h_spans;
             dry_signal = h_signal;
@@ -2351,6 +2400,7 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
         out["BarriersCounted"] = (long long)ex.barriers_counted;
         out["GemvChains"] = (long long)ex.gemv_chains;
         out["GemvClaimed"] = (long long)ex.gemv_claimed;
+        out["GemmXcdOrdered"] = (long long)ex.gemm_xcd_ordered;
         out["BarriersWidened"] = (long long)ex.barriers_widened;
         out["IterationSync"] = (long long)ex.iteration_sync;
         out["NumCounters"] = (long long)ex.dry_counters;
@@ -2369,6 +2419,10 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
                 j["Group"] = (long long)st.index;
                 j["NumTasks"] = (long long)n_tasks;
                 j["Chain"] = (long long)g.chain;
+                if (ex.dry_ops.size() > (size_t)g.op_begin && ex.dry_ops[(size_t)g.op_begin].kind == arkmi::DEV_GEMM) {
+                    j["XcdRound"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.xcd_round;
+                    j["XcdBand"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.xcd_band;
+                }
                 j["Claimed"] = g.claim >= 0;
                 Json waits = Json::array();
                 for (int w = 0; w < g.n_waits; ++w) {

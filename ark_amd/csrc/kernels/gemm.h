@@ -55,6 +55,8 @@ struct GemmDesc {
     // tile t; both leave their fp32 accumulators in `partial` and count in `arrivals[t]`; the one
     // that arrives second adds the other's and finishes the tile.  Nobody waits.
     int32_t split_k;           // 1 or 2
+    // XCD-aware order of the tiles (gemm_tile): xcd_round > 0 turns it on
+    int32_t xcd_round, xcd_band;
     int32_t pad_;
     float *partial;            // [tiles][2 halves][MT * NT][512 threads] x 4 floats
     unsigned int *arrivals;    // [tiles], zero between uses
@@ -174,7 +176,30 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     const int tiles_per_batch = d.tiles_m * d.tiles_n;
     const int bidx = task / tiles_per_batch;
     const int t2 = task % tiles_per_batch;
-    const int tm = t2 / d.tiles_n, tn = t2 % d.tiles_n;
+    int tm = t2 / d.tiles_n, tn = t2 % d.tiles_n;
+    if (d.xcd_round > 0) {
+        // Workgroups go to the chip's eight XCDs round robin and every XCD has its own L2, so
+        // with tasks dealt in tile order an XCD's concurrent tiles are strewn over the whole
+        // output and its L2 fetches nearly all of A.  Here the tile index is permuted so that the
+        // R / 8 tiles an XCD works on at a time form a block of xcd_band tile rows by
+        // R / (8 xcd_band) tile columns (R = xcd_round: the tasks that run at once).  The tiles are
+        // ordered in bands of xcd_band rows, column by column inside a band; task index t2 of a
+        // full round takes position ((round * 8 + xcd) * R / 8 + number within the XCD) of that
+        // order; the tasks of an incomplete last round keep their positions.  (The host sets this
+        // only where tiles_m is a multiple of xcd_band and task t runs on workgroup t mod R.)
+        const int R = d.xcd_round, per = R >> 3, bm = d.xcd_band;
+        int p = t2;
+        if (t2 < (tiles_per_batch / R) * R) {
+            const int r = t2 / R, q = t2 - r * R;
+            p = (r * 8 + (q & 7)) * per + (q >> 3);
+        }
+        const int band = bm * d.tiles_n, b = p / band, w = p - b * band;
+        tn = w / bm;
+        tm = b * bm + (w - tn * bm);
+        // the tile's own index from here on: partial tiles, arrivals and the ops fused behind
+        // the matmul go by it
+        task = bidx * tiles_per_batch + tm * d.tiles_n + tn;
+    }
     const int m0 = tm * BM, n0 = tn * BN;
 
     const int bn = bidx / d.batch_c, bc = bidx % d.batch_c;

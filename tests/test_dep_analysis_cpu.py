@@ -180,3 +180,50 @@ def test_consecutive_skinny_matmuls_form_one_stream():
     assert a["GemvChains"] == 2 and a["GemvClaimed"] == 2
     assert [(s["Chain"], s["Claimed"]) for s in _tasks_steps(a)] == [
         (2, True), (-1, False), (0, False), (3, True), (-1, False), (-1, False), (0, False)]
+
+
+def _tile_of(t2, tiles_m, tiles_n, xcd_round, band):
+    """The tile that task index t2 computes in the XCD-aware order, restated from the rule: tiles
+    ordered in bands of `band` rows, column by column; a task of a full round of `xcd_round` tasks
+    takes position ((round * 8 + xcd) * xcd_round / 8 + number within the XCD), xcd = t2 mod 8."""
+    p = t2
+    if t2 < (tiles_m * tiles_n // xcd_round) * xcd_round:
+        r, q = divmod(t2, xcd_round)
+        p = (r * 8 + q % 8) * (xcd_round // 8) + q // 8
+    b, w = divmod(p, band * tiles_n)
+    return b * band + w % band, w // band
+
+
+def test_matmul_tiles_in_xcd_aware_order():
+    """compile() orders the tiles of the decoder layer's matmuls so that the tiles one XCD (task
+    index mod 8) works on at a time form a compact block: every tile is still computed exactly once,
+    and the 32 (or 16) concurrent tiles of an XCD span band x (n / band) tiles instead of being
+    strewn over all tile rows."""
+    m = Model()
+    blk = llama.TransformerBlock(m, 4096, 32, 11008, "bf16")
+    x, f, mask = m.tensor([1, 2048, 4096], "bf16"), m.tensor([1, 2048, 1, 128], "bf16"), m.tensor([1, 1, 2048, 2048], "bf16")
+    blk.forward(x, f, mask, fused=True, causal=True)
+    plan = _plan(m)
+    a = plan_analysis(plan, 0)
+    gemms = [s for s in _tasks_steps(a) if "XcdRound" in s]
+    assert a["GemmXcdOrdered"] == len(gemms) == 6  # q, k, v, wo, the gate/up pair, w2
+    infos = json.loads(plan)["TaskInfos"]
+    for s in gemms:
+        assert s["XcdRound"] > 0 and s["XcdRound"] % 8 == 0
+        cfg = infos[s["Group"]]["Ops"][0]["Config"]
+        tm_, tn_ = cfg["TileShapeMNK"][:2]
+        tiles = s["NumTasks"] // cfg.get("SplitK", 1)
+        out_n = 4096 if tiles in (128, 256) else 2 * 11008
+        tiles_n = out_n // tn_
+        tiles_m = tiles // tiles_n
+        assert tiles_m * tiles_n == tiles and tiles_m % s["XcdBand"] == 0
+        where = [_tile_of(t, tiles_m, tiles_n, s["XcdRound"], s["XcdBand"]) for t in range(tiles)]
+        assert sorted(where) == [(i, j) for i in range(tiles_m) for j in range(tiles_n)]
+        per = s["XcdRound"] // 8
+        for xcd in range(8):
+            mine = where[xcd:s["XcdRound"]:8]
+            assert len(mine) == per
+            assert len({i for i, _ in mine}) == s["XcdBand"] and len({j for _, j in mine}) == per // s["XcdBand"]
+    # (waits and signals go by task index: a matmul that takes part in the dependency counters keeps
+    # the plain order)
+    assert plan_analysis(plan, 1)["GemmXcdOrdered"] < len(gemms)
