@@ -1131,6 +1131,7 @@ struct Executor {
     GemvSeqEntry *d_gemv_seq = nullptr;
     unsigned int *d_gemv_claims = nullptr;
     size_t gemv_claim_bytes = 0;
+    int attn_xcd_ordered = 0;               // attention ops whose tasks run in the XCD-aware order
     int gemm_xcd_ordered = 0;               // matmuls whose tiles run in the XCD-aware order
     int barriers_widened = 0;               // barriers over part of the grid made full-grid for claimed stretches
     int gemv_claimed = 0;                   // skinny matmuls (or runs of them) whose stretches are claimed at run time
@@ -1630,6 +1631,7 @@ struct Executor {
         // form a compact block (gemm_tile).  The tasks stay on their workgroups; the tile a task
         // computes changes, and the ops fused behind the matmul follow it.  ARKMI_GEMM_XCD=0: off.
         gemm_xcd_ordered = 0;
+        attn_xcd_ordered = 0;
         {
             const char *xe = getenv("ARKMI_GEMM_XCD");
             // (a workgroup-local sync in place of a barrier rests on task t of both ops running on
@@ -1638,6 +1640,19 @@ struct Executor {
             // only itself across iterations still computes the same tile on the same workgroup)
             const bool on = !(xe && atoi(xe) == 0) && !trace_enabled && barriers_local == 0 &&
                             !(iteration_sync == 1 && iteration_local_across_groups);
+            // (the attention op likewise: the query blocks an XCD works on at a time then belong to
+            // the same few heads)
+            for (DevTaskGroup &g : h_groups) {
+                DevOp &op0 = ops[(size_t)g.op_begin];
+                if (!on || op0.kind != DEV_ATTN || g.n_waits > 0 || g.signal_begin >= 0) continue;
+                if (g.proc_b != 0 || g.proc_s != 1 || g.proc_cur != 0 || g.task_b != 0 || g.task_s != 1 || g.gran != 1)
+                    continue;
+                AttnDesc &d = op0.attn;
+                const int total = d.batch * d.heads * d.q_blocks, round = std::min(total, (int)g.proc_e);
+                if (g.task_e != total || g.proc_e % 8 != 0 || round % 8 != 0 || round < 16) continue;
+                d.xcd_round = round;
+                ++attn_xcd_ordered;
+            }
             for (DevTaskGroup &g : h_groups) {
                 DevOp &op0 = ops[(size_t)g.op_begin];
                 if (!on || op0.kind != DEV_GEMM || op0.gemm.dtype == 0) continue;
@@ -2401,6 +2416,7 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
         out["GemvChains"] = (long long)ex.gemv_chains;
         out["GemvClaimed"] = (long long)ex.gemv_claimed;
         out["GemmXcdOrdered"] = (long long)ex.gemm_xcd_ordered;
+        out["AttnXcdOrdered"] = (long long)ex.attn_xcd_ordered;
         out["BarriersWidened"] = (long long)ex.barriers_widened;
         out["IterationSync"] = (long long)ex.iteration_sync;
         out["NumCounters"] = (long long)ex.dry_counters;

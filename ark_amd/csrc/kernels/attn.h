@@ -41,6 +41,10 @@ struct AttnDesc {
     int32_t causal;   // 1: key j is visible to query i iff j <= i + (seq_k - seq_q)
     int32_t dtype;    // 1 fp16, 2 bf16
     int32_t q_blocks; // ceil(seq_q / 128)
+    // > 0: the tasks that run at once (task t on workgroup t mod xcd_round); the task index is then
+    // permuted so that the query blocks an XCD (t mod 8) works on at a time belong to the same few
+    // heads, whose K and V its L2 then fetches once instead of every XCD fetching every head's
+    int32_t xcd_round;
 };
 
 constexpr int kAttnD = 128;        // head dimension
@@ -67,7 +71,18 @@ inline int attn_num_tasks(int batch, int heads, int seq_q) {
 }
 
 template <typename T>
-__device__ __forceinline__ void attn_task(const AttnDesc &d, int task, const Slot &s) {
+__device__ __forceinline__ void attn_task(const AttnDesc &d, int task_in, const Slot &s) {
+    int task = task_in;
+    if (d.xcd_round > 0) {
+        // position ((round * 8 + xcd) * R / 8 + number within the XCD) of the (head, query block)
+        // order below for a task of a full round of R; t and t + R keep their distance, so the
+        // pairing of long and short query blocks on a workgroup stands
+        const int R = d.xcd_round, total = d.batch * d.heads * d.q_blocks;
+        if (task < (total / R) * R) {
+            const int r = task / R, q = task - r * R;
+            task = (r * 8 + (q & 7)) * (R >> 3) + (q >> 3);
+        }
+    }
     const int tid = s.tid, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int qi = lane & 15, g = lane >> 4;

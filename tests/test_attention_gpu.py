@@ -120,3 +120,32 @@ def test_attention_causal_first_row_is_first_value(oracle):
     v = make(oracle, (1, 256, 2, 128), dtype, 97)
     got = run_attention(q, k, v, 0.0883883, True, dtype)
     assert np.array_equal(got[0, 0], v[0, 0])
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("shape", [(1, 2048, 2048, 32), (2, 1024, 1024, 12), (1, 640, 640, 8)])
+def test_attention_same_bits_in_both_task_orders(oracle, monkeypatch, causal, shape):
+    """The XCD-aware order of the attention tasks (the query blocks an XCD works on at a time belong
+    to the same few heads) changes which workgroup computes a (head, query block), not how: the same
+    bits as in plain task order (ARKMI_GEMM_XCD=0), on the decoder layer's shape (two full rounds of
+    256 tasks), with a partial last round (192 tasks in a round of 192; 40 tasks), and a sampled
+    head against float64."""
+    from ark_amd import Model, plan_analysis
+    b, sq, sk, h = shape
+    dtype = "bf16"
+    q = make(oracle, (b, sq, h, 128), dtype, 91)
+    k = make(oracle, (b, sk, h, 128), dtype, 92)
+    v = make(oracle, (b, sk, h, 128), dtype, 93)
+    scale = 1.0 / np.sqrt(128.0)
+    m = Model()
+    tq, tk, tv = m.tensor(q.shape, dtype), m.tensor(k.shape, dtype), m.tensor(v.shape, dtype)
+    m.attention(tq, tk, tv, scale, causal=causal)
+    assert plan_analysis(m.plan(arch="ROCM_950", num_processors=256))["AttnXcdOrdered"] == 1
+    got = run_attention(q, k, v, scale, causal, dtype)
+    monkeypatch.setenv("ARKMI_GEMM_XCD", "0")
+    plain = run_attention(q, k, v, scale, causal, dtype)
+    assert np.array_equal(got, plain)
+    hs = [0, h - 1]
+    exact = exact_attention(oracle, q[:, :, hs], k[:, :, hs], v[:, :, hs], scale, causal, dtype)
+    emx, erms = errors(oracle, exact, np.ascontiguousarray(got[:, :, hs]), dtype)
+    assert emx <= 1e-2 and erms <= 1e-2, (emx, erms)
