@@ -1645,11 +1645,14 @@ struct Executor {
             for (DevTaskGroup &g : h_groups) {
                 DevOp &op0 = ops[(size_t)g.op_begin];
                 if (!on || op0.kind != DEV_ATTN || g.n_waits > 0 || g.signal_begin >= 0) continue;
-                if (g.proc_b != 0 || g.proc_s != 1 || g.proc_cur != 0 || g.task_b != 0 || g.task_s != 1 || g.gran != 1)
+                // (task t on the (t mod n_procs)-th processor of a range that starts at a multiple of 8)
+                if (g.proc_b % 8 != 0 || g.proc_s != 1 || g.proc_cur != g.proc_b || g.task_b != 0 || g.task_s != 1 ||
+                    g.gran != 1)
                     continue;
                 AttnDesc &d = op0.attn;
-                const int total = d.batch * d.heads * d.q_blocks, round = std::min(total, (int)g.proc_e);
-                if (g.task_e != total || g.proc_e % 8 != 0 || round % 8 != 0 || round < 16) continue;
+                const int n_procs = g.proc_e - g.proc_b;
+                const int total = d.batch * d.heads * d.q_blocks, round = std::min(total, n_procs);
+                if (g.task_e != total || n_procs % 8 != 0 || round % 8 != 0 || round < 16) continue;
                 d.xcd_round = round;
                 ++attn_xcd_ordered;
             }
@@ -1658,9 +1661,10 @@ struct Executor {
                 if (!on || op0.kind != DEV_GEMM || op0.gemm.dtype == 0) continue;
                 GemmDesc &d = op0.gemm;
                 if (d.batch_total != 1 || g.n_waits > 0 || g.signal_begin >= 0) continue;  // (waits go by task index)
-                if (g.proc_b != 0 || g.proc_s != 1 || g.proc_cur != 0 || g.task_b != 0 || g.task_s != 1 || g.gran != 1)
+                if (g.proc_b % 8 != 0 || g.proc_s != 1 || g.proc_cur != g.proc_b || g.task_b != 0 || g.task_s != 1 ||
+                    g.gran != 1)
                     continue;
-                const int n_procs = g.proc_e, tiles = d.tiles_m * d.tiles_n;
+                const int n_procs = g.proc_e - g.proc_b, tiles = d.tiles_m * d.tiles_n;
                 const int round = std::min(tiles, n_procs);  // tiles in flight at once
                 if (n_procs % 8 != 0 || tiles % 8 != 0 || round % 8 != 0 || round < 16) continue;
                 if (g.task_e != tiles * (d.split_k == 2 ? 2 : 1)) continue;

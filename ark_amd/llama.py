@@ -111,14 +111,36 @@ class Attention:
     def params(self):
         return {"wq": self.wq, "wk": self.wk, "wv": self.wv, "wo": self.wo}
 
-    def forward(self, x, freqs_cis, mask, fused=False, residual=None, causal=False):
+    def forward(self, x, freqs_cis, mask, fused=False, residual=None, causal=False, pair_on=None):
         """causal=True (fused path only) states that `mask` is the causal mask: the
         attention then runs as one op that applies it arithmetically, skips the key
-        blocks above the diagonal and needs no transposes."""
+        blocks above the diagonal and needs no transposes.  pair_on=P (fused path only): the
+        number of processors the plan is made for; see below."""
         m = self.m
         bsz, seqlen, _ = x.shape
         h, hd = self.n_heads, self.head_dim
-        if fused and freqs_cis is not None:
+        # With 256x256 tiles one projection of this size may fill exactly half of the processors:
+        # the query and key projections, which do not depend on each other, are then placed side by
+        # side (ProcessorRange, the reference's planner-context mechanism,
+        # python/ark/planner.py:110-170), and the loop kernel, which drops the barrier between
+        # independent ops, runs them at the same time on full-size tiles instead of one after the
+        # other on half-size ones.
+        rows = bsz * seqlen
+        side_by_side = (fused and freqs_cis is not None and pair_on is not None and pair_on % 2 == 0
+                        and rows % 256 == 0 and self.dim % 256 == 0
+                        and (rows // 256) * (self.dim // 256) == pair_on // 2)
+        if side_by_side:
+            big = {"NumWarps": 8, "SramBytes": 131072, "TileShapeMNK": [256, 256, 64], "NumTasks": pair_on // 2}
+            half = pair_on // 2
+            with m.planner_context(processor_range=[0, half], sync=False):
+                with m.planner_context(config=big):
+                    yq = linear(m, x, self.wq)
+                xq = m.rope(m.reshape(yq, [bsz, seqlen, h, hd]), freqs_cis)
+            with m.planner_context(processor_range=[half, pair_on], sync=False):
+                with m.planner_context(config=big):
+                    yk = linear(m, x, self.wk)
+                xk = m.rope(m.reshape(yk, [bsz, seqlen, h, hd]), freqs_cis)
+        elif fused and freqs_cis is not None:
             # the rotation rides on the projections' tiles (a tile spans whole heads)
             with m.planner_context(sync=False):
                 xq = m.rope(m.reshape(linear(m, x, self.wq), [bsz, seqlen, h, hd]), freqs_cis)
@@ -179,7 +201,9 @@ class TransformerBlock:
         p.update({"feed_forward." + k: v for k, v in self.feed_forward.params().items()})
         return p
 
-    def forward(self, x, freqs_cis, mask, fused=False, causal=False):
+    def forward(self, x, freqs_cis, mask, fused=False, causal=False, pair_on=None):
+        """pair_on=P (fused path): the plan is made for P processors; projections that fill half of
+        them on full-size tiles are placed side by side (Attention.forward)."""
         m = self.m
         nx = rmsnorm(m, x, self.attention_norm, self.dtype, self.norm_eps, fused)
         if not fused:
@@ -187,7 +211,7 @@ class TransformerBlock:
             nh = rmsnorm(m, h, self.ffn_norm, self.dtype, self.norm_eps, fused)
             return m.add(h, self.feed_forward.forward(nh, fused))
         # the residual adds ride on the output projections' tiles
-        h = self.attention.forward(nx, freqs_cis, mask, fused, residual=x, causal=causal)
+        h = self.attention.forward(nx, freqs_cis, mask, fused, residual=x, causal=causal, pair_on=pair_on)
         nh = rmsnorm(m, h, self.ffn_norm, self.dtype, self.norm_eps, fused)
         return self.feed_forward.forward(nh, fused, residual=h)
 

@@ -249,15 +249,22 @@ def config_c4(torch, Model, Executor, inp, cpu):
 
 
 def config_c5(torch, np, Model, Executor, llama, inp, cpu):
-    names = {False: "reference_composition", True: "fused_ops", "attention": "fused_ops_attention_op"}
+    names = {False: "reference_composition", True: "fused_ops", "attention": "fused_ops_attention_op",
+             "side_by_side": "fused_ops_attention_op_qk_side_by_side"}
     out = {}
-    for fused in (False, True, "attention"):
+    num_cu = torch.cuda.get_device_properties(0).multi_processor_count
+    for fused in (False, True, "attention", "side_by_side"):
+        # "side_by_side": the attention-op plan with the query and key projections on full-size tiles
+        # on the two halves of the processors at the same time (one kernel per op cannot do that)
+        key, pair_on = fused, None
+        if fused == "side_by_side":
+            fused, pair_on = "attention", num_cu
         m = Model()
         blk = llama.TransformerBlock(m, 4096, 32, 11008, "bf16")
         tx = m.tensor([1, 2048, 4096], "bf16")
         tf = m.tensor([1, 2048, 1, 128], "bf16")
         tm = m.tensor([1, 1, 2048, 2048], "bf16")
-        blk.forward(tx, tf, tm, fused=bool(fused), causal=(fused == "attention"))
+        blk.forward(tx, tf, tm, fused=bool(fused), causal=(fused == "attention"), pair_on=pair_on)
         vals = {"x": inp.normal("hidden", tx.shape, torch.bfloat16)}
         feeds = [(tx, vals["x"]),
                  (tf, torch.from_numpy(llama.precompute_freqs_cis(128, 2048)).cuda().bfloat16()),
@@ -272,7 +279,7 @@ def config_c5(torch, np, Model, Executor, llama, inp, cpu):
         loop_us, info = _resident_us(torch, Executor, plan, 10, feeds)
         one_us, sep_us = _oneshot_and_separate_us(torch, Executor, plan, 10, feeds)
         counters = None
-        if fused == "attention":
+        if fused == "attention" and pair_on is None:
             # the same plan with its grid barriers replaced by dependency counters (off by default)
             os.environ["ARKMI_DEP_COUNTERS"] = "1"
             try:
@@ -283,7 +290,7 @@ def config_c5(torch, np, Model, Executor, llama, inp, cpu):
         # full (unskipped) attention counts 897.7 GFLOP; the attention op skips the masked key blocks
         fl = 863.3e9 if fused == "attention" else 897.7e9
         base = None
-        if cpu and fused == "attention":
+        if cpu and fused == "attention" and pair_on is None:
             from oracle import ark_oracle as O
             host = {k: v.view(torch.int16).cpu().numpy().view("uint16") for k, v in vals.items() if v.dtype == torch.bfloat16}
             xs = host["x"][0, :16]
@@ -299,13 +306,15 @@ def config_c5(torch, np, Model, Executor, llama, inp, cpu):
                               "oracle Q and output projections and the SwiGLU FFN on 16 of the 2048 positions "
                               "(the K/V projections and the attention itself are left out of the CPU sample)")
         del feeds, vals
-        out[names[fused]] = _block(
+        out[names[key]] = _block(
             "C5 Llama-2-7B decoder layer, seq 2048, d 4096, 32 heads x 128, SwiGLU 11008, bf16, RoPE 10000, causal ("
             + {False: "the reference's op-by-op composition", True: "fused ops, matmul/softmax attention",
-               "attention": "fused ops, attention as one op; flop count with masked key blocks skipped"}[fused] + ")",
+               "attention": "fused ops, attention as one op; flop count with masked key blocks skipped",
+               "side_by_side": "fused ops, attention as one op, query and key projections side by side on "
+                               "256x256 tiles; flop count with masked key blocks skipped"}[key] + ")",
             "mfma", fl, one_us, loop_us, sep_us, info, base)
         if counters:
-            out[names[fused]]["with_dependency_counters"] = counters
+            out[names[key]]["with_dependency_counters"] = counters
     return out
 
 

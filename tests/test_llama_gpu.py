@@ -116,24 +116,34 @@ def test_decoder_layer_small(oracle, dtype, fused):
     assert mx <= TOL and rms <= TOL, (mx, rms)
 
 
-@pytest.mark.parametrize("fused", [False, True, "attention"])
+@pytest.mark.parametrize("fused", [False, True, "attention", "side_by_side"])
 def test_decoder_layer_full_size_sampled_rows(oracle, fused):
     """Llama-2-7B layer shape: seq 2048, d 4096, 32 heads x 128, SwiGLU 11008,
     bf16, RoPE base 10000, causal mask.  The oracle evaluates 24 sampled query
-    positions against the whole sequence's keys and values."""
+    positions against the whole sequence's keys and values.  "side_by_side": the attention-op
+    plan with the query and key projections on 256x256 tiles on the two halves of the processors
+    at the same time (no barrier between them)."""
     from ark_amd import Model
+    pair_on = None
+    if fused == "side_by_side":
+        fused, pair_on = "attention", 256
     dtype, seq, dim, heads, hidden = "bf16", 2048, 4096, 32, 11008
     m = Model()
     blk, vals, x, freqs, mask = _layer_case(oracle, m, seq, dim, heads, hidden, dtype, 400)
     tx = m.tensor([1, seq, dim], dtype)
     tf = m.tensor([1, seq, 1, dim // heads], dtype)
     tm = m.tensor([1, 1, seq, seq], dtype)
-    out = blk.forward(tx, tf, tm, fused=fused, causal=(fused == "attention"))
+    out = blk.forward(tx, tf, tm, fused=fused, causal=(fused == "attention"), pair_on=pair_on)
     feeds = {tx: x, tf: oracle.to_storage(freqs, dtype), tm: oracle.to_storage(mask, dtype)}
     if fused == "attention":
         del feeds[tm]  # the attention op applies the causal mask itself: no mask tensor in the plan
     feeds.update({t: vals[name] for name, t in blk.params().items()})
     got, info = _run(m, feeds, out)
+    if pair_on:
+        import json
+        from ark_amd import plan_schedule
+        groups = json.loads(m.plan(device_id=0))["ProcessorGroups"]
+        assert [g["ProcessorRange"] for g in groups[1:3]] == [[0, 128], [128, 256]]
     pick = np.sort(np.random.default_rng(9).choice(seq, 24, replace=False))
     pick[0], pick[-1] = 0, seq - 1
     ref = R.transformer_block(oracle, x, vals, freqs, mask, heads, dtype, q_rows=pick)
