@@ -350,6 +350,15 @@ def timeline(torch, np, Model, Executor, llama, prng, which):
         plan = m.plan(device_id=0)
         cases.append(("C5 fused ops with the attention op, grid barriers", plan, feeds, {}))
         cases.append(("C5 fused ops with the attention op, dependency counters", plan, feeds, {"ARKMI_DEP_COUNTERS": "1"}))
+        # the same layer with the query and key projections side by side (same parameter tensors
+        # by name, so the same seeded values)
+        m2 = Model()
+        blk2 = llama.TransformerBlock(m2, 4096, 32, 11008, "bf16")
+        tx2, tf2, tm2 = m2.tensor([1, 2048, 4096], "bf16"), m2.tensor([1, 2048, 1, 128], "bf16"), m2.tensor([1, 1, 2048, 2048], "bf16")
+        blk2.forward(tx2, tf2, tm2, fused=True, causal=True, pair_on=torch.cuda.get_device_properties(0).multi_processor_count)
+        by_name = {name: v for (name, _), (_, v) in zip(blk.params().items(), feeds[2:])}
+        feeds2 = [(tx2, feeds[0][1]), (tf2, feeds[1][1])] + [(t, by_name[name]) for name, t in blk2.params().items()]
+        cases.append(("C5 fused ops with the attention op, query and key projections side by side", m2.plan(device_id=0), feeds2, {}))
     for title, plan, feeds, env in cases:
         names = {ti["Id"]: "+".join(o["Type"] for o in ti["Ops"]) for ti in _json.loads(plan)["TaskInfos"]}
         sched = [(names[st["Args"][-1]] if st["Kind"] == "TaskSeq" else "B") for st in plan_schedule(plan)["Steps"]]
