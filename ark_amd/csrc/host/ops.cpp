@@ -153,9 +153,9 @@ static Json rocm950_config(const ModelOp &op, int num_cu) {
         }
         // Largest tile that divides the padded problem and still gives every CU
         // a task; otherwise the dividing tile with the most tasks.
-        const bool tall = mnk[0] > mnk[1];
-        const int64_t cand[4][2] = {{256, 256}, {tall ? 256 : 128, tall ? 128 : 256},
-                                    {tall ? 128 : 256, tall ? 256 : 128}, {128, 128}};
+        // (of the two half-size tiles the 256-row one first: measured faster than 128x256 on
+        // the same problem, 161 against 171 us on 4096^3 and 9 us per decoder layer)
+        const int64_t cand[4][2] = {{256, 256}, {256, 128}, {128, 256}, {128, 128}};
         int64_t tm = 0, tn = 0;
         for (const auto &c : cand) {
             // the one tile shape of a transposed input and of FP32 operands

@@ -119,18 +119,26 @@ def test_decoder_layer_replaces_every_barrier():
     waits = {w["ProducerGroup"]: w for w in g["attn"]["Waits"]}
     assert sorted(waits) == [g["q"]["Group"], g["k"]["Group"], g["v"]["Group"]]
     qb_count = 2048 // 128
+    # (a projection's row blocks are its tile rows: bm rows each, one signal per tile column)
+    bm, bn = _cfg(plan, g["q"]["Group"])["TileShapeMNK"][:2]
     for t in range(g["attn"]["NumTasks"]):
         bh, qb = divmod(t, qb_count)
         if bh >= 16:  # the upper half of the heads runs its query blocks backwards
             qb = qb_count - 1 - qb
-        assert tuple(waits[g["q"]["Group"]]["Spans"][t]) == (qb, qb), t
-        assert tuple(waits[g["k"]["Group"]]["Spans"][t]) == (0, qb), t
-        assert tuple(waits[g["v"]["Group"]]["Spans"][t]) == (0, qb), t
-    # every projection block expects one signal per tile column (4096 / 256 = 16 tiles)
-    assert all(w["Expect"] == 16 for w in waits.values())
-    # the output projection reads all heads of its rows: 128 query rows = 32 attention tasks per block
+        first, last = qb * 128 // bm, (qb * 128 + 127) // bm
+        assert tuple(waits[g["q"]["Group"]]["Spans"][t]) == (first, last), t
+        assert tuple(waits[g["k"]["Group"]]["Spans"][t]) == (0, last), t
+        assert tuple(waits[g["v"]["Group"]]["Spans"][t]) == (0, last), t
+    assert all(w["Expect"] == 4096 // bn for w in waits.values())
+    # the output projection reads all heads of its rows: 128 query rows = 32 attention tasks per
+    # attention row block, and a tile row of bm_o rows spans bm_o / 128 of them
     (w,) = g["wo"]["Waits"]
     assert w["ProducerGroup"] == g["attn"]["Group"] and w["Expect"] == 32
+    bm_o = _cfg(plan, g["wo"]["Group"])["TileShapeMNK"][0]
+    tiles_n_o = 4096 // _cfg(plan, g["wo"]["Group"])["TileShapeMNK"][1]
+    for t, (lo, hi) in enumerate(w["Spans"]):
+        r0 = (t // tiles_n_o) * bm_o
+        assert (lo, hi) == (r0 // 128, (r0 + bm_o - 1) // 128), t
     # the down projection needs the SwiGLU rows of its tile and the residual it adds
     assert sorted(w["ProducerGroup"] for w in g["down"]["Waits"]) == sorted([g["wo"]["Group"], g["swiglu"]["Group"]])
     assert "SignalMap" not in g["down"]
