@@ -118,7 +118,7 @@ def test_counters_across_commands_and_relaunch(oracle, monkeypatch):
         ex.stop()
 
 
-@pytest.mark.parametrize("fused", [True, "attention"])
+@pytest.mark.parametrize("fused", [True, "attention", "side_by_side"])
 def test_decoder_layer_with_counters(oracle, fused, monkeypatch):
     """The fused Llama decoder layer (RMSNorm -> projections with the rotation on their tiles ->
     attention -> output projection with the residual -> RMSNorm -> SwiGLU -> down projection with the
@@ -134,9 +134,11 @@ def test_decoder_layer_with_counters(oracle, fused, monkeypatch):
         tx = m.tensor([1, seq, dim], dtype)
         tf = m.tensor([1, seq, 1, dim // heads], dtype)
         tm = m.tensor([1, 1, seq, seq], dtype)
-        out = blk.forward(tx, tf, tm, fused=bool(fused), causal=(fused == "attention"))
+        side_by_side = fused == "side_by_side"  # query and key projections on the two halves of the processors
+        kind = "attention" if side_by_side else fused
+        out = blk.forward(tx, tf, tm, fused=bool(kind), causal=(kind == "attention"), pair_on=256 if side_by_side else None)
         feeds = {tx: x, tf: oracle.to_storage(freqs, dtype), tm: oracle.to_storage(mask, dtype)}
-        if fused == "attention":
+        if kind == "attention":
             del feeds[tm]
         feeds.update({t: vals[name] for name, t in blk.params().items()})
         (got,), info = _run(m, feeds, [out], iters=2)
