@@ -1417,6 +1417,55 @@ struct Executor {
         }
         num_dev_steps = (int)steps.size();
 
+        // ---- row ops whose input another op reads afterwards: fetch it through the caches ---------
+        // (RowOpDesc::in_read_again; ARKMI_ROW_CACHED_INPUT=0: every row op streams its input)
+        {
+            const char *env = getenv("ARKMI_ROW_CACHED_INPUT");
+            const bool on = !(env && atoi(env) == 0);
+            auto input_of = [&](const Json &op_json, Access &out) {
+                std::vector<Access> v;
+                const Json &reads = op_json.at("ReadTensors");
+                if (reads.size() == 0) return false;
+                add_access(v, reads.at((size_t)0), false, op_json.at("Type").as_string(), false);
+                if (v.empty()) return false;
+                out = v[0];
+                return true;
+            };
+            auto same_bytes = [](const Access &x, const Access &y) {
+                return x.buffer == y.buffer && x.begin < y.end && y.begin < x.end;
+            };
+            for (size_t si = 0; on && si < sched.steps.size(); ++si) {
+                if (sched.steps[si].is_barrier || dev_step_of[si] < 0) continue;
+                const DevTaskGroup &g = h_groups[(size_t)steps[(size_t)dev_step_of[si]].index];
+                const Json &task_ops = task_infos.at((size_t)sched.steps[si].task_info).at("Ops");
+                for (int o = 0; o < g.op_count; ++o) {
+                    DevOp &op = ops[(size_t)(g.op_begin + o)];
+                    Access in;
+                    if (op.kind != DEV_ROW || op.row.red_len > 0 || !input_of(task_ops.at((size_t)o), in)) continue;
+                    // the accesses that follow this op: the later ops of its task, then the later steps
+                    std::vector<Access> later;
+                    for (size_t o2 = (size_t)o + 1; o2 < task_ops.size(); ++o2) {
+                        Json one = Json::object();
+                        Json arr = Json::array();
+                        arr.push_back(task_ops.at(o2));
+                        one["Ops"] = arr;
+                        auto a = accesses_of(one);
+                        later.insert(later.end(), a.begin(), a.end());
+                    }
+                    for (size_t sj = si + 1; sj < sched.steps.size(); ++sj)
+                        if (!sched.steps[sj].is_barrier) {
+                            auto a = step_accesses(sj);
+                            later.insert(later.end(), a.begin(), a.end());
+                        }
+                    for (const Access &y : later) {
+                        if (!same_bytes(in, y)) continue;
+                        op.row.in_read_again = y.write ? 0 : 1;  // (overwritten first: nobody reads these values again)
+                        break;
+                    }
+                }
+            }
+        }
+
         // ---- dependency counters in place of full-grid barriers --------------------------------
         // Task groups since the last barrier that stays form a window.  A full-grid barrier inside
         // the window is replaced by a workgroup sync when every hazard between a group behind it
@@ -2439,6 +2488,16 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
                 j["Group"] = (long long)st.index;
                 j["NumTasks"] = (long long)n_tasks;
                 j["Chain"] = (long long)g.chain;
+                if (ex.dry_ops.size() >= (size_t)(g.op_begin + g.op_count)) {
+                    Json again = Json::array();
+                    bool any_row = false;
+                    for (int o = 0; o < g.op_count; ++o) {
+                        const arkmi::DevOp &op = ex.dry_ops[(size_t)(g.op_begin + o)];
+                        any_row = any_row || op.kind == arkmi::DEV_ROW;
+                        again.push_back((long long)(op.kind == arkmi::DEV_ROW ? op.row.in_read_again : 0));
+                    }
+                    if (any_row) j["InputReadAgain"] = again;
+                }
                 if (ex.dry_ops.size() > (size_t)g.op_begin && ex.dry_ops[(size_t)g.op_begin].kind == arkmi::DEV_GEMM) {
                     j["XcdRound"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.xcd_round;
                     j["XcdBand"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.xcd_band;

@@ -235,3 +235,28 @@ def test_matmul_tiles_in_xcd_aware_order():
     # (waits and signals go by task index: a matmul that takes part in the dependency counters keeps
     # the plain order)
     assert plan_analysis(plan, 1)["GemmXcdOrdered"] < len(gemms)
+
+
+def test_row_ops_whose_input_is_read_again():
+    """A row op whose input another op of the plan reads afterwards fetches it through the caches
+    (the later reader then finds it there); the last reader, and an op whose input is overwritten
+    before anybody reads it again, stream it."""
+    m = Model()
+    x, y = m.tensor([16384, 4096], "fp16"), m.tensor([16384, 4096], "fp16")
+    w = m.tensor([4096], "fp32")
+    m.reduce_sum(x, -1)
+    m.softmax(x)
+    m.rmsnorm(x, w, 1e-6)          # the last reader of x
+    m.reduce_sum(y, -1)            # y is overwritten next, before anybody reads it
+    m.softmax(x, output=y)
+    m.rmsnorm(y, w, 1e-6)          # reads the new y; nobody after it
+    a = plan_analysis(_plan(m), 0)
+    assert [s["InputReadAgain"] for s in _tasks_steps(a)] == [[1], [1], [1], [0], [0], [0]]
+    # (x is read once more by the fifth op, so the third is not its last reader)
+    m = Model()
+    x = m.tensor([16384, 4096], "fp16")
+    m.reduce_sum(x, -1)
+    m.softmax(x)
+    m.rmsnorm(x, m.tensor([4096], "fp32"), 1e-6)
+    a = plan_analysis(_plan(m), 0)
+    assert [s["InputReadAgain"] for s in _tasks_steps(a)] == [[1], [1], [0]]

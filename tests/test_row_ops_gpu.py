@@ -137,3 +137,36 @@ def test_errors():
         ops.softmax(x)
     with pytest.raises(ValueError):
         ops.softmax(torch.zeros(4, 8))
+
+
+def test_row_ops_over_one_tensor_cached_and_streamed_inputs_agree(oracle, monkeypatch):
+    """reduce_sum, softmax and RMSNorm over the same X in one plan: the first two fetch X through
+    the caches because a later op reads it again, the last one streams it.  The load policy changes
+    no value: the same bits with every input streamed (ARKMI_ROW_CACHED_INPUT=0), and the softmax
+    against the oracle."""
+    from ark_amd import Model, Executor
+    dtype = "fp16"
+    x = make(oracle, (2048, 4096), dtype, seed=77, dist="normal")
+    w = np.random.default_rng(5).uniform(0.5, 1.5, 4096).astype(np.float32)
+
+    def run():
+        m = Model()
+        tx, tw = m.tensor([2048, 4096], dtype), m.tensor([4096], "fp32")
+        outs = [m.reduce_sum(tx, -1), m.softmax(tx), m.rmsnorm(tx, tw, 1e-6)]
+        ex = Executor(m.plan(device_id=0)).compile()
+        ex.tensor_write(tx, x)
+        ex.tensor_write(tw, w)
+        ex.launch()
+        ex.run(2)
+        ex.wait()
+        got = [ex.tensor_read(t) for t in outs]
+        ex.stop()
+        return got
+
+    a = run()
+    monkeypatch.setenv("ARKMI_ROW_CACHED_INPUT", "0")
+    b = run()
+    for p, q in zip(a, b):
+        assert np.array_equal(p, q)
+    ref = oracle.softmax(x, dtype)
+    assert np.abs(oracle.to_f32(a[1], dtype) - oracle.to_f32(ref, dtype)).max() <= 1e-3
