@@ -1,9 +1,13 @@
 """Planner, runtime, modules and state-dict files of the `ark` surface.
 
-Follows python/ark/planner.py:110-230, runtime.py:15-168, module.py:13-89, init.py:10-17 and
-serialize.py:8-28: same names, same state machine, same messages for misuse.
+Behaviour to match: python/ark/planner.py:110-230 (plan objects and the planner),
+runtime.py:27-168 (the three-state life cycle), module.py:13-89 (module trees and state
+dicts), init.py:10-17 and serialize.py:8-28 (state-dict files).  The runtime is written as a
+transition table, the module as one ordered registry of named members, and state-dict files
+are read by an unpickler that constructs numpy arrays and plain containers only.
 """
 import copy as _copy
+import io
 import json
 import logging
 import pickle
@@ -100,188 +104,271 @@ class Executor(_x.Executor):
         self._copy(tensor._tensor, ndarray.ctypes.data, ndarray.nbytes, True, stream=stream)
 
 
-class _RuntimeState:
+_log = logging.getLogger("ark")
+
+
+class _Live:
+    """What outlives a Runtime object: the process-wide runtime and the one executor that may
+    hold device memory at a time."""
     runtime = None
     executor = None
 
+    @classmethod
+    def retire_executor(cls):
+        ex, cls.executor = cls.executor, None
+        if ex is not None and not ex.destroyed():
+            ex.destroy()
+
 
 class Runtime:
-    """Init -> launch() -> LaunchedNotRunning -> run() -> Running -> wait() -> LaunchedNotRunning;
-    stop() keeps the executor for another launch(), reset() destroys it."""
+    """The life cycle of the global model on one device.
+
+    Three states; each public call looks its (state, call) pair up in `_TABLE`, which names the
+    step to take and the state to end in.  A pair mapped to `_refuse` raises, one mapped to
+    `_skip` logs and returns None.
+
+        state               launch        run          wait        barrier     stop
+        Init                build+start   refuse       skip        refuse      skip
+        LaunchedNotRunning  skip          start iters  skip        barrier     halt
+        Running             skip          refuse       complete    refuse      halt
+
+    `stop()` halts the kernel but leaves the state at LaunchedNotRunning with the executor (and
+    its device memory) alive, so tensors stay readable; `reset()` returns to Init and frees it.
+    """
 
     class State(Enum):
         Init = 0
         LaunchedNotRunning = 1
         Running = 2
 
+    # -- the steps ---------------------------------------------------------------------------
+    def _build_and_start(self, plan=None, device_id=0, stream=0, loop_mode=True):
+        if plan is None:
+            plan = Planner(device_id).plan()
+        if _Live.executor is not None and not _Live.executor.destroyed():
+            _log.warning("Destroying an old executor")
+        _Live.retire_executor()
+        self.executor = _Live.executor = Executor(device_id, stream, "ArkRuntime", str(plan), loop_mode)
+        self.executor.compile()
+        self.executor.launch()
+
+    def _start_iterations(self, iter=1, non_blocking=False):
+        self.executor.run(iter)
+        return non_blocking
+
+    def _complete(self):
+        self.executor.wait()
+
+    def _barrier(self):
+        self.executor.barrier()
+
+    def _halt(self):
+        return self.executor.stop()
+
+    def _refuse(self, *args, **kwargs):
+        _log.error("ARK runtime is not launched")
+        raise RuntimeError("ARK runtime is not launched")
+
+    _SKIP_NOTES = {
+        "launch": "Runtime is already launched, skip launching",
+        "wait": "ARK runtime is not running, skip waiting",
+        "stop": "ARK runtime is never launched, skip stopping",
+    }
+
+    _I, _L, _R = State.Init, State.LaunchedNotRunning, State.Running
+    _TABLE = {
+        (_I, "launch"): (_build_and_start, _L), (_L, "launch"): (None, _L), (_R, "launch"): (None, _R),
+        (_I, "run"): (_refuse, _I), (_L, "run"): (_start_iterations, _R), (_R, "run"): (_refuse, _R),
+        (_I, "wait"): (None, _I), (_L, "wait"): (None, _L), (_R, "wait"): (_complete, _L),
+        (_I, "barrier"): (_refuse, _I), (_L, "barrier"): (_barrier, _L), (_R, "barrier"): (_refuse, _R),
+        (_I, "stop"): (None, _I), (_L, "stop"): (_halt, _L), (_R, "stop"): (_halt, _L),
+    }
+    del _I, _L, _R
+
+    def _step(self, call, *args, **kwargs):
+        action, after = Runtime._TABLE[(self.state, call)]
+        if action is None:
+            _log.warning(Runtime._SKIP_NOTES[call])
+            return None
+        out = action(self, *args, **kwargs)
+        self.state = after
+        return out
+
+    # -- the public calls --------------------------------------------------------------------
     @staticmethod
     def get_runtime():
-        if _RuntimeState.runtime is None:
-            _RuntimeState.runtime = Runtime()
-        return _RuntimeState.runtime
+        return _Live.runtime if _Live.runtime is not None else Runtime()
 
     def __init__(self):
         self.executor = None
         self.state = Runtime.State.Init
-        _RuntimeState.runtime = self
+        _Live.runtime = self   # the newest runtime is the one tensors talk to
 
-    def __del__(self):
-        try:
-            self.reset()
-        except Exception:  # interpreter shutdown: the library may already be gone
-            pass
+    def launched(self):
+        return self.state is not Runtime.State.Init
+
+    def running(self):
+        return self.state is Runtime.State.Running
+
+    def launch(self, plan=None, device_id=0, stream=0, loop_mode=True):
+        """Plans the global model (unless a plan is given), allocates and starts the kernel."""
+        self._step("launch", plan, device_id, stream, loop_mode)
+
+    def run(self, iter=1, non_blocking=False):
+        if not self._step("run", iter, non_blocking):
+            self.wait()
+
+    def wait(self):
+        self._step("wait")
+
+    def barrier(self):
+        self._step("barrier")
+
+    def stop(self):
+        """Halts the kernel; elapsed milliseconds since the launch, or None if never launched."""
+        return self._step("stop")
+
+    def reset(self):
+        """Back to Init: the kernel halted, the executor and its device memory released."""
+        if self.launched():
+            self.stop()
+        ex, self.executor = self.executor, None
+        if ex is not None:
+            if ex is _Live.executor:
+                _Live.retire_executor()
+            elif not ex.destroyed():
+                ex.destroy()
+        self.state = Runtime.State.Init
 
     def __enter__(self):
         return self
 
-    def __exit__(self, exc_type, exc_val, exc_tb):
+    def __exit__(self, *exc):
         self.reset()
 
-    def launched(self):
-        return self.state in (Runtime.State.LaunchedNotRunning, Runtime.State.Running)
-
-    def running(self):
-        return self.state == Runtime.State.Running
-
-    def launch(self, plan=None, device_id=0, stream=0, loop_mode=True):
-        if self.launched():
-            logging.warning("Runtime is already launched, skip launching")
-            return
-        plan = Planner(device_id).plan() if plan is None else plan
-        if self.state == Runtime.State.Init:
-            old = _RuntimeState.executor
-            if old is not None and not old.destroyed():
-                logging.warning("Destroying an old executor")
-                old.destroy()
-            _RuntimeState.executor = Executor(device_id, stream, "ArkRuntime", str(plan), loop_mode)
-            self.executor = _RuntimeState.executor
-            self.executor.compile()
-        self.executor.launch()
-        self.state = Runtime.State.LaunchedNotRunning
-
-    def run(self, iter=1, non_blocking=False):
-        if self.state != Runtime.State.LaunchedNotRunning:
-            logging.error("ARK runtime is not launched")
-            raise RuntimeError("ARK runtime is not launched")
-        self.state = Runtime.State.Running
-        self.executor.run(iter)
-        if not non_blocking:
-            self.wait()
-
-    def barrier(self):
-        if self.state != Runtime.State.LaunchedNotRunning:
-            logging.error("ARK runtime is not launched")
-            raise RuntimeError("ARK runtime is not launched")
-        self.executor.barrier()
-
-    def wait(self):
-        if self.state != Runtime.State.Running:
-            logging.warning("ARK runtime is not running, skip waiting")
-            return
-        self.executor.wait()
-        self.state = Runtime.State.LaunchedNotRunning
-
-    def stop(self):
-        """Stops the kernel; returns the elapsed milliseconds.  launch() starts it again."""
-        if not self.launched():
-            logging.warning("ARK runtime is never launched, skip stopping")
-            return None
-        elapsed = self.executor.stop()
-        self.state = Runtime.State.LaunchedNotRunning
-        return elapsed
-
-    def reset(self):
-        if self.launched():
-            self.stop()
-        if self.executor is not None:
-            if not self.executor.destroyed():
-                self.executor.destroy()
-            self.executor = None
-        self.state = Runtime.State.Init
+    def __del__(self):
+        try:
+            self.reset()
+        except Exception:  # interpreter shutdown: the native library may be gone already
+            pass
 
 
 class Module:
-    """Tree of modules and parameters; attribute assignment registers them."""
+    """A node of a model tree.  Assigning a Module or a Parameter to an attribute enters it in
+    the node's registry under the attribute's name (assigning again replaces the entry);
+    `sub_modules` and `parameters` are the two views of that registry, in order of entry."""
 
-    def __init__(self):
-        self.sub_modules = {}
-        self.parameters = {}
+    def _members(self):
+        return self.__dict__.setdefault("_registry", {})
 
     def __setattr__(self, name, value):
-        if isinstance(value, Module):
-            self.register_module(name, value)
-        elif isinstance(value, Parameter):
-            self.register_parameter(name, value)
-        super().__setattr__(name, value)
+        if isinstance(value, (Module, Parameter)):
+            self._members()[name] = value
+        object.__setattr__(self, name, value)
 
-    def __call__(self, *args, **kwargs):
-        return self.forward(*args, **kwargs)
+    @property
+    def sub_modules(self):
+        return {k: v for k, v in self._members().items() if isinstance(v, Module)}
+
+    @property
+    def parameters(self):
+        return {k: v for k, v in self._members().items() if isinstance(v, Parameter)}
 
     def register_module(self, name, module):
         if not isinstance(module, Module):
             raise TypeError("module must be a Module")
-        self.sub_modules[name] = module
+        self._members()[name] = module
 
     def register_parameter(self, name, param):
         if not isinstance(param, Parameter):
             raise TypeError("param must be a Parameter")
-        self.parameters[name] = param
+        self._members()[name] = param
+
+    def _walk(self, prefix):
+        """(dotted name, Parameter) of every parameter below this node: sub-modules first, in
+        order of entry, then the node's own parameters."""
+        for name, sub in self.sub_modules.items():
+            yield from sub._walk(f"{prefix}{name}.")
+        for name, p in self.parameters.items():
+            yield prefix + name, p
 
     def params_dict(self, prefix=""):
-        out = {}
-        for name, sub in self.sub_modules.items():
-            if sub is not None:
-                out.update(sub.params_dict(prefix=prefix + name + "."))
-        for name, p in self.parameters.items():
-            out[prefix + name] = p
-        return out
-
-    def load_state_dict(self, state_dict, prefix=""):
-        """Copies arrays to the parameters' device memory; the runtime must be launched."""
-        unused = set(state_dict.keys())
-        for name, p in self.params_dict(prefix).items():
-            p.from_numpy(state_dict[name])
-            unused.remove(name)
-        if unused:
-            logging.warning(f"{len(unused)} unused parameter(s) in state_dict")
+        return dict(self._walk(prefix))
 
     def state_dict(self, prefix=""):
-        return {k: v.to_numpy() for k, v in self.params_dict(prefix).items()}
+        """Every parameter read back as a numpy array (shapes only before the launch)."""
+        return {name: p.to_numpy() for name, p in self._walk(prefix)}
+
+    def load_state_dict(self, state_dict, prefix=""):
+        """Writes the arrays to the parameters' device memory (after `Runtime.launch()`); a
+        parameter without an array is a KeyError, arrays without a parameter are reported."""
+        used = set()
+        for name, p in self._walk(prefix):
+            p.from_numpy(state_dict[name])
+            used.add(name)
+        extra = len(set(state_dict) - used)
+        if extra:
+            _log.warning("%d unused parameter(s) in state_dict", extra)
 
     def forward(self, *args, **kwargs):
-        ...
+        """What the module appends to the global model; a subclass defines it."""
+        return None
 
     def backward(self, *args, **kwargs):
-        ...
+        """Placeholder, as in the reference: nothing here differentiates."""
+        return None
+
+    def __call__(self, *args, **kwargs):
+        return self.forward(*args, **kwargs)
 
 
 def init():
-    """Drops the global model, destroys a live executor and reads the ARK_* environment again."""
+    """Starts over: the `ARK_*` environment is read again, the global model is dropped, a live
+    executor is destroyed and the runtime returns to Init."""
     from .._lib import lib, check
     check(lib().arkmi_init())
     Model.reset()
-    ex = _RuntimeState.executor
-    if ex is not None:
-        if not ex.destroyed():
-            ex.destroy()
-    _RuntimeState.executor = None
-    if _RuntimeState.runtime is not None:
-        _RuntimeState.runtime.executor = None
-        _RuntimeState.runtime.state = Runtime.State.Init
+    _Live.retire_executor()
+    rt = _Live.runtime
+    if rt is not None:
+        rt.executor, rt.state = None, Runtime.State.Init
+
+
+# ---- state-dict files -------------------------------------------------------------------------
+# The file format is the reference's: one pickled dict of numpy arrays.  Unpickling a file runs
+# whatever callables it names, so the reader resolves only the few that numpy arrays and plain
+# containers are made of and refuses every other global.
+_ARRAY_GLOBALS = {
+    ("numpy", "ndarray"), ("numpy", "dtype"),
+    ("numpy.core.multiarray", "_reconstruct"), ("numpy._core.multiarray", "_reconstruct"),
+    ("numpy.core.multiarray", "scalar"), ("numpy._core.multiarray", "scalar"),
+    ("numpy.core.numeric", "_frombuffer"), ("numpy._core.numeric", "_frombuffer"),
+    ("collections", "OrderedDict"),
+}
+
+
+class _ArrayUnpickler(pickle.Unpickler):
+    def find_class(self, module, name):
+        if (module, name) not in _ARRAY_GLOBALS:
+            raise pickle.UnpicklingError(f"state-dict files hold numpy arrays only; refusing {module}.{name}")
+        return super().find_class(module, name)
 
 
 def save(state_dict, state_dict_file_path):
-    """Writes a state dict in the reference's file format (a pickled dict of numpy arrays)."""
+    """Writes `{name: numpy array}` to a file `load()` (and the reference's) can read."""
     if not isinstance(state_dict, dict):
-        logging.warning("Invalid state_dict saved to %s", state_dict_file_path)
+        _log.warning("Invalid state_dict saved to %s", state_dict_file_path)
+    payload = pickle.dumps(state_dict, protocol=4)
+    _ArrayUnpickler(io.BytesIO(payload)).load()   # nothing is written that load() would refuse
     with open(state_dict_file_path, "wb") as f:
-        pickle.dump(state_dict, f)
+        f.write(payload)
 
 
 def load(state_dict_file_path):
-    """Reads a file save() wrote.  Unpickling runs code from the file: load your own files only."""
+    """Reads a state-dict file without running code from it: a file that names anything but
+    numpy's array constructors raises `pickle.UnpicklingError`."""
     with open(state_dict_file_path, "rb") as f:
-        state_dict = pickle.load(f)
+        state_dict = _ArrayUnpickler(f).load()
     if not isinstance(state_dict, dict):
-        logging.warning("Invalid state_dict file")
+        _log.warning("Invalid state_dict file")
     return state_dict

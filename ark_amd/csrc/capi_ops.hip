@@ -1,4 +1,6 @@
 // Stand-alone launchers of the op bodies (one kernel launch per op).
+#include <atomic>
+
 #include "host_common.h"
 #include "host/ops.hpp"
 #include "kernels/gemm.h"
@@ -234,14 +236,21 @@ extern "C" int arkmi_gemv_plan(int m, int n, int k, int num_tasks, int *num_task
 
 namespace arkmi {
 
-// Validates the arguments of a skinny matmul, fills the descriptor and launches it with
-// `workspace` (counters first, then partials) of at least the planned size.
-static void launch_gemv(int dtype, const void *x, const void *w, void *y, int m, int n, int k, int64_t ldx,
-                        int64_t ldw, int64_t ldy, int num_tasks, void *workspace, hipStream_t st) {
+constexpr int kMaxDevices = 64;
+
+// What a skinny matmul asks of its operands; checked before anything is launched or written.
+static void check_gemv_operands(const void *x, const void *w, const void *y, int n, int k, int64_t ldx, int64_t ldw,
+                                int64_t ldy) {
     if (!x || !w || !y) ARKMI_FAIL(ARKMI_INVALID_USAGE, "null tensor pointer");
     if (ldx < k || ldw < n || ldy < n) ARKMI_FAIL(ARKMI_INVALID_USAGE, "leading dimension too small");
     if ((n % 8) || (ldx % 8) || (ldw % 8) || ((uintptr_t)x & 15) || ((uintptr_t)w & 15))
         ARKMI_FAIL(ARKMI_UNSUPPORTED, "operands must be 16-byte aligned with N and leading dimensions % 8 == 0");
+}
+
+// Fills the descriptor of a skinny matmul whose operands passed check_gemv_operands and launches
+// it with `workspace` (counters first, then partials) of at least the planned size.
+static void launch_gemv(int dtype, const void *x, const void *w, void *y, int m, int n, int k, int64_t ldx,
+                        int64_t ldw, int64_t ldy, int num_tasks, void *workspace, hipStream_t st) {
     GemvDesc d{};
     d.x = x; d.w = w; d.y = y;
     d.m = m; d.n = n; d.k = k;
@@ -250,12 +259,15 @@ static void launch_gemv(int dtype, const void *x, const void *w, void *y, int m,
     gemv_partition(d, num_tasks);
     d.counters = static_cast<unsigned int *>(workspace);
     d.partial = reinterpret_cast<float *>(static_cast<char *>(workspace) + gemv_counter_bytes(d.n_blocks));
-    static bool attr_set[2] = {false, false};
+    // (set once per type and device; two threads that both find it unset both set it, which is harmless)
+    static std::atomic<bool> attr_set[2][kMaxDevices];
     const int ti = dtype == ARKMI_FP16 ? 0 : 1;
+    const int dev = current_device();
+    if (dev < 0 || dev >= kMaxDevices) ARKMI_FAIL(ARKMI_UNSUPPORTED, "device index ", dev, " out of range");
     const void *kern = ti == 0 ? (const void *)gemv_kernel<f16> : (const void *)gemv_kernel<bf16>;
-    if (!attr_set[ti]) {
+    if (!attr_set[ti][dev].load(std::memory_order_acquire)) {
         ARKMI_HIP(hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, kGemvLdsBytes));
-        attr_set[ti] = true;
+        attr_set[ti][dev].store(true, std::memory_order_release);
     }
     int ntasks = d.num_tasks;
     void *args[] = {&d, &ntasks};
@@ -270,19 +282,19 @@ static void launch_gemv(int dtype, const void *x, const void *w, void *y, int m,
 constexpr size_t kGemvStaticBytes = (size_t)16 << 20;
 static __device__ __align__(256) unsigned char g_gemv_scratch[kGemvStaticBytes];
 
-constexpr int kMaxDevices = 64;
-static void *g_gemv_scratch_ptr[kMaxDevices];  // per device, null until resolved
+// per device, null until resolved (threads that race to resolve a device store the same address)
+static std::atomic<void *> g_gemv_scratch_ptr[kMaxDevices];
 
 static void *gemv_static_workspace() {
     const int dev = current_device();
     if (dev < 0 || dev >= kMaxDevices) ARKMI_FAIL(ARKMI_UNSUPPORTED, "device index ", dev, " out of range");
-    if (!g_gemv_scratch_ptr[dev]) {
-        void *p = nullptr;
+    void *p = g_gemv_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
         ARKMI_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(g_gemv_scratch)));
         if (!p) ARKMI_FAIL(ARKMI_GPU_ERROR, "the library's static workspace has no address on device ", dev);
-        g_gemv_scratch_ptr[dev] = p;
+        g_gemv_scratch_ptr[dev].store(p, std::memory_order_release);
     }
-    return g_gemv_scratch_ptr[dev];
+    return p;
 }
 
 // Zero fill by a kernel: callers may be under stream capture, where memset nodes are avoided.
@@ -304,6 +316,7 @@ extern "C" int arkmi_gemv(int dtype, const void *x, const void *w, void *y, int 
             throw Error(rc, arkmi_last_error());
         if (!workspace || workspace_bytes < need)
             ARKMI_FAIL(ARKMI_INVALID_USAGE, "workspace of ", need, " bytes needed, got ", workspace_bytes);
+        check_gemv_operands(x, w, y, n, k, ldx, ldw, ldy);
         launch_gemv(dtype, x, w, y, m, n, k, ldx, ldw, ldy, num_tasks, workspace, (hipStream_t)stream);
     });
 }
@@ -321,6 +334,8 @@ extern "C" int arkmi_gemv_static(int dtype, const void *x, const void *w, void *
         if (need > kGemvStaticBytes)
             ARKMI_FAIL(ARKMI_UNSUPPORTED, "this shape needs ", need, " bytes of workspace; the library's static workspace holds ",
                        kGemvStaticBytes, " (use arkmi_gemv with a workspace of your own)");
+        // a call that is going to be refused leaves the shared workspace alone
+        check_gemv_operands(x, w, y, n, k, ldx, ldw, ldy);
         void *ws = gemv_static_workspace();
         hipStream_t st = (hipStream_t)stream;
         // the array keeps whatever the last call left: the arrival counters must start at zero

@@ -1473,6 +1473,9 @@ struct Executor {
         // read of rows whose writers signal counters the reader waits on.  A hazard that is
         // neither keeps the last barrier ahead of the reader.  ARKMI_DEP_COUNTERS=1 turns this on.
         barriers_counted = 0;
+        // a hazard across a candidate barrier was accepted as workgroup-local: task t of both
+        // groups must then keep computing tile t (no permuted tile order below)
+        bool counted_relies_on_local = false;
         std::vector<DevWait> h_waits;
         std::vector<int32_t> h_spans, h_signal;
         size_t n_counters = 0;
@@ -1529,7 +1532,11 @@ struct Executor {
                         for (size_t ia = 0; ia < dg[(size_t)xi].acc.size(); ++ia)
                             for (size_t ib = 0; ib < dg[(size_t)yi].acc.size(); ++ib) {
                                 const Access &ax = dg[(size_t)xi].acc[ia], &ay = dg[(size_t)yi].acc[ib];
-                                if (!overlap(ax, ay) || local_pair(ax, ay)) continue;
+                                if (!overlap(ax, ay)) continue;
+                                if (local_pair(ax, ay)) {
+                                    counted_relies_on_local = true;
+                                    continue;
+                                }
                                 if (cover_with_counters(dg, xi, ax, yi, ay, arena, buffer_offset)) continue;
                                 if (getenv("ARKMI_DEBUG_BARRIERS"))
                                     fprintf(stderr, "no counters for steps %d -> %d: views '%s' (%s) vs '%s' (%s)\n",
@@ -1686,6 +1693,7 @@ struct Executor {
             // two groups across the iteration boundary, keep the plain order; a group that meets
             // only itself across iterations still computes the same tile on the same workgroup)
             const bool on = !(xe && atoi(xe) == 0) && !trace_enabled && barriers_local == 0 &&
+                            !(barriers_counted > 0 && counted_relies_on_local) &&
                             !(iteration_sync == 1 && iteration_local_across_groups);
             // (the attention op likewise: the query blocks an XCD works on at a time then belong to
             // the same few heads)

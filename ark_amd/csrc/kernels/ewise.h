@@ -394,7 +394,10 @@ __device__ __forceinline__ void ewise_cast_from(const EwiseDesc &d, int task, co
 
 // ---- embedding gather ---------------------------------------------------------------
 // out[n, c, h, :] = weight[idx[n, c, h], :] with negative indices counted from the end of
-// the table (ark/include/kernels/embedding.h:107-143).  One wave per output row: the
+// the table (ark/include/kernels/embedding.h:107-143).  An index outside [-num_emb, num_emb)
+// names no row: it is clamped to the nearest one (row 0 or the last), so that index data
+// from a user can never make the gather read outside the table; the reference reads
+// whatever lies there.  One wave per output row: the
 // index is a uniform load, the row moves as 16-byte vectors when both rows are aligned.
 struct EmbedDesc {
     const int32_t *idx;
@@ -417,6 +420,7 @@ __device__ __forceinline__ void embedding_task(const EmbedDesc &d, int task, con
     const int64_t h = row % d.dim_h, c = (row / d.dim_h) % d.dim_c, n = row / ((int64_t)d.dim_h * d.dim_c);
     int e = as_global(d.idx)[n * d.idx_s[0] + c * d.idx_s[1] + h * d.idx_s[2]];
     if (e < 0) e += d.num_emb;
+    e = min(max(e, 0), d.num_emb - 1);
     e = __builtin_amdgcn_readfirstlane(e);
     gptr<const char> src = as_global(static_cast<const char *>(d.weight)) + (int64_t)e * d.w_pitch * d.elem;
     gptr<char> dst = as_global(static_cast<char *>(d.out)) +

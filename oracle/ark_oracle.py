@@ -274,12 +274,16 @@ def cast(x, src, dst):
     return out
 
 
-def embedding(indices, weight):
+def embedding(indices, weight, clamp=False):
     """out[..., :] = weight[indices[...], :], negative indices counted from the end of the
     table (the host baseline of ark/ops/ops_embedding_test.cpp:11-41).  Pure data movement:
-    works on the storage bits of any type."""
+    works on the storage bits of any type.  An index outside [-rows, rows) has no meaning in the
+    reference (its baseline and its kernel both read outside the table); with `clamp` such an
+    index takes the nearest row after the wrap, which is what the device code here does."""
     idx = np.asarray(indices, dtype=np.int64)
     idx = np.where(idx < 0, idx + weight.shape[0], idx)
+    if clamp:
+        idx = np.clip(idx, 0, weight.shape[0] - 1)
     return np.ascontiguousarray(weight[idx])
 
 

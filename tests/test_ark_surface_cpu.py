@@ -254,3 +254,53 @@ def test_runtime_refuses_before_launch():
     assert rt.stop() is None
     rt.reset()
     assert rt.state == ark.Runtime.State.Init
+
+
+def test_load_refuses_a_pickle_that_names_other_globals(tmp_path):
+    import pickle
+
+    class _Payload:
+        def __reduce__(self):
+            return (print, ("code from the file ran",))
+
+    f = tmp_path / "bad.pkl"
+    f.write_bytes(pickle.dumps({"w": _Payload()}))
+    with pytest.raises(pickle.UnpicklingError, match="refusing"):
+        ark.load(str(f))
+    # arrays of every storage type the tensors use, nested containers and numpy scalars pass
+    sd = {"a": np.ones((2, 3), np.float32), "b": np.arange(4, dtype=np.int32),
+          "c": {"d": [np.float16(1.5), (1, 2.0, "s", None, True)]}}
+    g = str(tmp_path / "good.pkl")
+    ark.save(sd, g)
+    back = ark.load(g)
+    assert np.array_equal(back["a"], sd["a"]) and back["c"]["d"][0] == np.float16(1.5)
+    assert back["c"]["d"][1] == (1, 2.0, "s", None, True)
+
+
+def test_runtime_transition_table_is_total_and_matches_the_reference_life_cycle():
+    """Every (state, call) pair has an entry; the end states are the ones
+    python/ark/runtime.py:60-168 reaches (stop leaves LaunchedNotRunning, run refuses unless
+    launched and idle, wait/stop/launch in the wrong state are skipped)."""
+    S, T = ark.Runtime.State, ark.Runtime._TABLE
+    calls = ["launch", "run", "wait", "barrier", "stop"]
+    assert sorted(T, key=str) == sorted(((s, c) for s in S for c in calls), key=str)
+    ends = {(s, c): T[(s, c)][1] for s in S for c in calls}
+    assert ends[(S.Init, "launch")] == S.LaunchedNotRunning
+    assert ends[(S.LaunchedNotRunning, "run")] == S.Running
+    assert ends[(S.Running, "wait")] == S.LaunchedNotRunning
+    assert ends[(S.Running, "stop")] == ends[(S.LaunchedNotRunning, "stop")] == S.LaunchedNotRunning
+    refused = {k for k, (a, _) in T.items() if a is ark.Runtime._refuse}
+    assert refused == {(S.Init, "run"), (S.Init, "barrier"), (S.Running, "run"), (S.Running, "barrier")}
+    skipped = {k for k, (a, _) in T.items() if a is None}
+    assert skipped == {(S.LaunchedNotRunning, "launch"), (S.Running, "launch"), (S.Init, "wait"),
+                       (S.LaunchedNotRunning, "wait"), (S.Init, "stop")}
+    assert all(ends[k] == k[0] for k in refused | skipped)
+
+
+def test_module_reassignment_and_a_module_without_forward():
+    m = _Mlp()
+    first = m.up
+    m.up = _Linear(64, 32)                       # replaces the entry, keeps its position
+    assert list(m.sub_modules) == ["up", "down"] and m.sub_modules["up"] is not first
+    assert list(m.params_dict()) == ["up.weight", "down.weight", "bias"]   # sub-modules first
+    assert ark.Module()() is None

@@ -260,3 +260,29 @@ def test_row_ops_whose_input_is_read_again():
     m.rmsnorm(x, m.tensor([4096], "fp32"), 1e-6)
     a = plan_analysis(_plan(m), 0)
     assert [s["InputReadAgain"] for s in _tasks_steps(a)] == [[1], [1], [0]]
+
+
+def test_counted_barrier_with_a_local_hazard_keeps_the_plain_tile_order():
+    """rmsnorm(x); y = a @ w; y + rmsnorm(x) with the add cut into the matmul's 256x256 tiles: with
+    counters on, the barrier ahead of the add goes because its hazard with the RMSNorm is counted
+    and its hazard with the matmul is local to a workgroup (task t of both covers tile t).  That
+    second half rests on the matmul computing tile t in task t, so the XCD-aware permutation of
+    its tiles must stay off; without counters the barrier stays and the permutation is on."""
+    m = Model()
+    x, a, w = (m.tensor([4096, 4096], "fp16") for _ in range(3))
+    n = m.rmsnorm(x)
+    m.add(m.matmul(a, w), n)
+    plan = json.loads(_plan(m))
+    add_cfg = plan["TaskInfos"][2]["Ops"][0]["Config"]
+    add_cfg["Tile"], add_cfg["NumTasks"] = [256, 256], 256
+    plan["ProcessorGroups"][2]["ResourceGroups"][0]["TaskGroups"][0]["TaskRange"] = [0, 256]
+    plan = json.dumps(plan)
+    on = plan_analysis(plan, 1)
+    assert [s["Kind"] for s in on["Steps"]] == ["Tasks", "Tasks", "LocalSync", "Tasks"]
+    assert on["BarriersCounted"] == 1 and on["BarriersLocal"] == 0
+    norm, mm, add = _tasks_steps(on)
+    assert [w_["ProducerGroup"] for w_ in add["Waits"]] == [norm["Group"]]   # nothing waits for the matmul
+    assert mm["XcdRound"] == 0 and on["GemmXcdOrdered"] == 0
+    off = plan_analysis(plan, 0)
+    assert [s["Kind"] for s in off["Steps"]] == ["Tasks", "Tasks", "Barrier", "Tasks"]
+    assert _tasks_steps(off)[1]["XcdRound"] == 256

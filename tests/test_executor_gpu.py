@@ -776,6 +776,22 @@ def test_embedding(oracle, dtype):
     assert np.array_equal(got, oracle.embedding(idx, w))
 
 
+def test_embedding_index_outside_the_table_is_clamped(oracle):
+    """Indices a table of 100 rows has no row for (100, 101, 2**31 - 1, -101, -2**31): the reference
+    reads outside the table there; here they take the last or the first row and never leave it."""
+    from ark_amd import Model
+    num_emb, dim = 100, 256
+    idx = np.array([[0, 99, 100, 101, 2**31 - 1, -1, -100, -101, -2**31, 7]], dtype=np.int32)
+    w = make(oracle, (num_emb, dim), "fp16", 14, "uniform")
+    m = Model()
+    ti, tw = m.tensor(idx.shape, "int32"), m.tensor(w.shape, "fp16")
+    out = m.embedding(ti, tw)
+    (got,), ex, _ = run_model(m, {ti: idx, tw: w}, [out])
+    want = oracle.embedding(idx, w, clamp=True)
+    assert np.array_equal(want[0, [2, 3, 4]], np.stack([w[99]] * 3)) and np.array_equal(want[0, [7, 8]], np.stack([w[0]] * 2))
+    assert np.array_equal(got, want)
+
+
 def test_embedding_ragged_rows_and_other_ops_in_one_plan(oracle):
     """A table whose rows are not whole 16-byte vectors (scalar path), a 1-D index vector, and a
     matmul on the gathered rows in the same plan."""
