@@ -233,13 +233,13 @@ static Json rocm950_config(const ModelOp &op, int num_cu) {
         return c;
     }
     if (t == "Attention") {
-        // one task = 128 query positions of one (batch, head); K and V blocks are
-        // double-buffered in LDS (must match kernels/attn.h)
+        // one task = 128 query positions of one (batch, head); steps of 128 keys, K and V
+        // tiles of 32 KB each, double-buffered in LDS (must match kernels/attn.h)
         const Dims &qs = op.read_tensors()[0]->shape();
         if (qs[3] != 128) ARK_ERR(PlanError, "the attention body supports head_dim 128, got ", qs[3]);
         Json c = Json::object();
         c["NumWarps"] = kWarps950;
-        c["SramBytes"] = 2 * 64 * ((128 * 2 + 16) + (128 * 2 + 32));
+        c["SramBytes"] = 2 * 2 * 128 * (128 * 2);
         c["NumTasks"] = (long long)(qs[0] * qs[2] * div_up(qs[1], 128));
         return c;
     }

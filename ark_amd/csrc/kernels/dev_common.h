@@ -144,6 +144,38 @@ __device__ __forceinline__ void drain_stores_then_barrier() {
 using lds_ptr = __attribute__((address_space(3))) char *;
 using lds_u32_ptr = __attribute__((address_space(3))) unsigned int *;
 
+// ---- global -> LDS direct loads ----------------------------------------------------
+// One wave-level load of 16 bytes per lane straight into LDS: lane i's bytes land at
+// dst + 16 i (dst is uniform; it travels in M0).  Written as an instruction of its own
+// rather than through the compiler's builtin: with loads of that builtin outstanding the
+// compiler puts s_waitcnt vmcnt(0) in front of every ds_read_b64_tr_b16 (it cannot tell
+// which LDS bytes a transposing read touches), which drains a ring's prefetch several times
+// per tile in every layout that reads through the transposing instruction.  Completion is
+// tracked by hand with vmcnt waits, as it has to be for the builtin too.  M0 is put back:
+// the compiler owns that register.
+template <typename P>
+__device__ __forceinline__ void direct_load16(P src, lds_ptr dst) {
+    const uint32_t m0v = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
+    uint32_t keep;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(src), "s"(m0v)
+                 : "memory");
+}
+// The same with the address as a uniform base plus a 32-bit byte offset per lane.
+template <typename P>
+__device__ __forceinline__ void direct_load16_at(P base, uint32_t lane_bytes, lds_ptr dst) {
+    const uint32_t m0v = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
+    const uint64_t b = (uint64_t)base;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)b), hi = __builtin_amdgcn_readfirstlane((uint32_t)(b >> 32));
+    const uint64_t sb = ((uint64_t)hi << 32) | lo;
+    uint32_t keep;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(lane_bytes), "s"(sb), "s"(m0v)
+                 : "memory");
+}
+
 constexpr unsigned kSlotSyncSpinLimit = 1u << 26;  // polls before a slot barrier gives up waiting
 
 struct Slot {

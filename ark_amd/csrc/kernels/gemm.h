@@ -5,8 +5,8 @@
 // (2 x 4 wave grid) with v_mfma_f32_16x16x32 (at the chip's power limit that shape
 // sustains about 15 % more flops than 32x32x16: a quarter of the accumulator
 // traffic per instruction for half the flops).  A and B tiles of depth BK
-// travel from global memory straight into LDS (global_load_lds_dwordx4, no
-// staging registers, no LDS store instructions) into a ring of S stage
+// travel from global memory straight into LDS (global_load_lds_dwordx4 through
+// direct_load16, no staging registers, no LDS store instructions) into a ring of S stage
 // buffers; the loads of the next S-1 tiles are in flight while the current one
 // is multiplied, and there is one workgroup barrier per tile.
 //
@@ -266,16 +266,12 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     auto issue_one = [&](int kt, int stage, int l) {
         const lds_ptr base = lds + stage * L::STAGE_BYTES + wave * kGemmLoadBytes;
         if (l < A_LD)
-            __builtin_amdgcn_global_load_lds((const ARKMI_GLOBAL void *)(a_src + l * a_step + kt * a_kstep),
-                                             (lds_void *)(base + l * 8 * kGemmLoadBytes), 16, 0, 0);
+            direct_load16(a_src + l * a_step + kt * a_kstep, base + l * 8 * kGemmLoadBytes);
         else if (DUAL_B)
-            __builtin_amdgcn_global_load_lds((const ARKMI_GLOBAL void *)(b_dual[l - A_LD] + kt * b_kstep),
-                                             (lds_void *)(base + L::A_BYTES + (l - A_LD) * 8 * kGemmLoadBytes), 16, 0,
-                                             0);
+            direct_load16(b_dual[l - A_LD] + kt * b_kstep, base + L::A_BYTES + (l - A_LD) * 8 * kGemmLoadBytes);
         else
-            __builtin_amdgcn_global_load_lds(
-                (const ARKMI_GLOBAL void *)(b_src + (l - A_LD) * b_step + kt * b_kstep),
-                (lds_void *)(base + L::A_BYTES + (l - A_LD) * 8 * kGemmLoadBytes), 16, 0, 0);
+            direct_load16(b_src + (l - A_LD) * b_step + kt * b_kstep,
+                          base + L::A_BYTES + (l - A_LD) * 8 * kGemmLoadBytes);
     };
     auto issue = [&](int kt, int stage) {
 #pragma unroll
@@ -536,14 +532,14 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     }
 
     // ---- epilogue: lane (m = lane%16, g = lane/16) holds C[m][4g .. 4g+3] of each 16x16 tile ----
+    // (store4 takes finished values: the epilogue hook or the gate/up product has been applied)
     const bool vec_ok = ((d.ldc & 3) == 0) && (((uintptr_t)d.c & 7) == 0) && ((d.c_bs[0] & 3) == 0) &&
                         ((d.c_bs[1] & 3) == 0);
     auto store4 = [&](int row, int col, float v0, float v1, float v2, float v3) {
         if (row >= d.store_m) return;
         gptr<T> p = C + (int64_t)row * d.ldc + col;
         if (vec_ok && col + 4 <= d.store_n) {
-            T o[4] = {from_f32<T>(epi(v0, row, col)), from_f32<T>(epi(v1, row, col + 1)),
-                      from_f32<T>(epi(v2, row, col + 2)), from_f32<T>(epi(v3, row, col + 3))};
+            T o[4] = {from_f32<T>(v0), from_f32<T>(v1), from_f32<T>(v2), from_f32<T>(v3)};
             u32x2 w;
             __builtin_memcpy(&w, o, 8);
             *(ARKMI_GLOBAL u32x2 *)p = w;
@@ -551,37 +547,75 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
             const float v[4] = {v0, v1, v2, v3};
 #pragma unroll
             for (int e = 0; e < 4; ++e)
-                if (col + e < d.store_n) p[e] = from_f32<T>(epi(v[e], row, col + e));
+                if (col + e < d.store_n) p[e] = from_f32<T>(v[e]);
         }
     };
-    if constexpr (DUAL_B) {
-        // accumulator tiles j and j + NT/2 of a wave hold the gate and the up product of the
-        // same 16 output columns
-        static_assert(NT % 2 == 0, "the gate/up pair needs an even number of column tiles per wave");
+    // The wave's output: NTO column tiles of 16 per 16-row strip.  For the gate/up pair accumulator
+    // tiles j and j + NT/2 of a wave hold the gate and the up product of the same 16 output columns.
+    static_assert(!DUAL_B || NT % 2 == 0, "the gate/up pair needs an even number of column tiles per wave");
+    constexpr int NTO = DUAL_B ? NT / 2 : NT;
+    const int col_w = DUAL_B ? tn * (BN / 2) + wn * (WTN / 2) : n0 + wn * WTN;  // the wave's first output column
+    const int out_n0 = DUAL_B ? tn * (BN / 2) : n0, out_bn = DUAL_B ? BN / 2 : BN;
+    auto value4 = [&](int i, int j, int row, int col, float *o) {
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const int row = m0 + wm * WTM + i * 16 + l16;
-#pragma unroll
-            for (int j = 0; j < NT / 2; ++j) {
-                const int col = tn * (BN / 2) + wn * (WTN / 2) + j * 16 + 4 * g4;
-                float o[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float g = acc[i][j][e], u = acc[i][j + NT / 2][e];
-                    o[e] = g / (1.f + __expf(-g)) * u;
-                }
-                store4(row, col, o[0], o[1], o[2], o[3]);
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (DUAL_B) {
+                const float g = acc[i][j][e], u = acc[i][j + NT / 2][e];
+                o[e] = g / (1.f + __expf(-g)) * u;
+            } else {
+                o[e] = epi(acc[i][j][e], row, col + e);
             }
         }
+    };
+    // Whole tiles of an aligned C go through LDS, strip by strip: a wave writes a strip of 16 rows
+    // x (16 NTO) columns (8 bytes per lane and column tile) into a window of its own and reads it
+    // back as 16 bytes per lane, LPR lanes to a row: every store instruction then writes whole row
+    // segments (128 bytes, a cache line, for four column tiles), where the accumulator layout by
+    // itself gives 32 bytes per row and instruction and the L2 writes some lines back more than
+    // once.  No barrier inside: a wave's LDS operations complete in order and the window is the
+    // wave's own (the stage ring is free: the K loop ended with every load landed and every wave
+    // past its last fragment read).
+    constexpr int SEG_B = NTO * 16 * 2;           // bytes of a strip's row
+    constexpr int SPITCH = SEG_B + 16;            // padded: rows 16 bytes apart modulo the bank span
+    constexpr int LPR = SEG_B / 16;               // lanes per row when reading back
+    constexpr int RPP = 64 / LPR;                 // rows per pass
+    constexpr bool kStaged = (64 % LPR == 0) && (RPP <= 16) && (16 % RPP == 0);
+    if (kStaged && vec_ok && (d.ldc & 7) == 0 && (((uintptr_t)d.c & 15) == 0) && (d.c_bs[0] & 7) == 0 &&
+        (d.c_bs[1] & 7) == 0 && m0 + BM <= d.store_m && out_n0 + out_bn <= d.store_n) {
+        const lds_ptr win = lds + wave * (2 * 16 * SPITCH);
+        const int rrow = lane / LPR, rchunk = lane % LPR;
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const lds_ptr buf = win + (i & 1) * 16 * SPITCH;
+            const int row = m0 + wm * WTM + i * 16 + l16;
+#pragma unroll
+            for (int j = 0; j < NTO; ++j) {
+                float o[4];
+                value4(i, j, row, col_w + j * 16 + 4 * g4, o);
+                T t[4] = {from_f32<T>(o[0]), from_f32<T>(o[1]), from_f32<T>(o[2]), from_f32<T>(o[3])};
+                u32x2 w;
+                __builtin_memcpy(&w, t, 8);
+                *(__attribute__((address_space(3))) u32x2 *)(buf + l16 * SPITCH + j * 32 + g4 * 8) = w;
+            }
+#pragma unroll
+            for (int p = 0; p < 16 / RPP; ++p) {
+                const int r = p * RPP + rrow;
+                const u32x4 v = *(const lds_u32x4 *)(buf + r * SPITCH + rchunk * 16);
+                *(ARKMI_GLOBAL u32x4 *)(C + (int64_t)(m0 + wm * WTM + i * 16 + r) * d.ldc + col_w + rchunk * 8) = v;
+            }
+        }
+        s.sync();  // the windows lie in the stage ring, which the next task (or another op body) fills
         return task;
     }
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int row = m0 + wm * WTM + i * 16 + l16;
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-            const int col = n0 + wn * WTN + j * 16 + 4 * g4;
-            store4(row, col, acc[i][j][0], acc[i][j][1], acc[i][j][2], acc[i][j][3]);
+        for (int j = 0; j < NTO; ++j) {
+            const int col = col_w + j * 16 + 4 * g4;
+            float o[4];
+            value4(i, j, row, col, o);
+            store4(row, col, o[0], o[1], o[2], o[3]);
         }
     }
     return task;

@@ -5,15 +5,20 @@ Headline (BASELINE config 2): row-wise fp16 ops on X[16384,4096] ~ N(0,1) — re
 the last axis, softmax, RMSNorm (weight ~ U(0.5,1.5), eps 1e-6), fp32 accumulation — planned
 by the Planner and executed inside ONE persistent loop kernel (Model -> plan JSON ->
 Executor).  The plan holds four X tensors (4 x 128 MiB, with outputs of their own) and walks
-them in turn, so the 256 MB Infinity Cache cannot serve repeated reads.  A "step" is one plan
-iteration: the three ops over each of the four X tensors (12 ops, 2.68 GB of algorithmic
-bytes).
+them in turn, so nothing of an X is left in the 256 MB Infinity Cache when its turn comes
+again.  Within a turn the three ops read the same X one after the other, and the second and
+third read may be served by that cache (the plan keeps X cacheable for them on purpose).  A
+"step" is one plan iteration: the three ops over each of the four X tensors (12 ops, 2.68 GB
+of algorithmic bytes).
 
 `value` is the whole-job throughput of the timed run of the resident loop kernel (host clock
 around run() + wait(), inputs already in HBM) in algorithmic GB/s.  `roofline` prices the
 loop kernel itself against 8 TB/s: the same plan launched in one-shot mode (the kernel runs
 its iterations and returns) under HIP events on the stream it is launched on, which is the
-dispatch `rocprofv3 --kernel-trace` reports.
+dispatch `rocprofv3 --kernel-trace` reports.  `roofline.frac` counts algorithmic bytes and so
+includes the cache-served re-reads; `roofline.frac_hbm_only` is the same plan with every op
+streaming its input from HBM (ARKMI_ROW_CACHED_INPUT=0), and `roofline.per_op` times each of
+the three ops alone over the four rotating X tensors, where no byte is read twice.
 
 `configs` holds the other BASELINE configurations (C1 GEMM, C3 SwiGLU FFN, C4 decode GEMV at
 batch 1 and 8, C5 decoder layer), each with the same kind of block: a HIP-event-timed one-shot
@@ -46,13 +51,14 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 
 
 def profiled_traffic_bytes_per_step():
-    """HBM bytes one step moves, as measured by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the
-    one-shot loop-kernel dispatch: read from the committed profile summary (not measured in
-    this run).  None when the summary is missing."""
+    """Bytes one step moves between the L2s and the fabric (Infinity Cache hits included; HBM
+    sees less), as measured by rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE on the one-shot
+    loop-kernel dispatch: read from the committed profile summary (not measured in this run).
+    None when the summary is missing."""
     path = os.path.join(ROOT, "profiles", "loop_kernel_rows_c2_pmc.txt")
     try:
         with open(path) as f:
-            m = re.search(r"^hbm_bytes_per_step:\s*(\d+)", f.read(), re.M)
+            m = re.search(r"^(?:fabric|hbm)_bytes_per_step:\s*(\d+)", f.read(), re.M)
         return (int(m.group(1)), "profiles/loop_kernel_rows_c2_pmc.txt") if m else (None, None)
     except OSError:
         return None, None
@@ -219,32 +225,46 @@ def config_c3(torch, Model, Executor, llama, inp, cpu):
 
 
 def config_c4(torch, Model, Executor, inp, cpu):
+    """Decode GEMV.  The headline block of a batch size walks TWO sets of the four matrices in turn
+    (810 MB, more than L2 and Infinity Cache hold), so every token step streams its 404.75 MB from
+    HBM; `one_weight_set` is the same token step over a single set, of which the 256 MB cache can
+    keep a part from one iteration to the next."""
     shapes = [("W_qkv", 4096, 12288), ("W_o", 4096, 4096), ("W_gate_up", 4096, 22016), ("W_down", 11008, 4096)]
     wbytes = float(sum(k * n * 2 for _, k, n in shapes))
     out = {}
     for bsz in (1, 8):
-        m = Model()
-        feeds, vals = [], []
-        for name, k, n in shapes:
-            tx, tw = m.tensor([bsz, k], "bf16"), m.tensor([k, n], "bf16")
-            m.matmul(tx, tw)
-            x, w = inp.normal(f"x_{name}_b{bsz}", tx.shape, torch.bfloat16), inp.normal(name, tw.shape, torch.bfloat16, 0.02)
-            feeds += [(tx, x), (tw, w)]
-            vals.append((x, w))
-        plan = m.plan(device_id=0)
-        loop_us, info = _resident_us(torch, Executor, plan, 50, feeds)
-        one_us, sep_us = _oneshot_and_separate_us(torch, Executor, plan, 50, feeds)
-        base = None
-        if cpu:
-            from oracle import ark_oracle as O
-            host = [(x.view(torch.int16).cpu().numpy().view("uint16"), w.view(torch.int16).cpu().numpy().view("uint16"))
-                    for x, w in vals]
-            base = _timed_cpu(lambda: [O.matmul(x, w, "bf16") for x, w in host], wbytes, "GB/s",
-                              f"oracle matmul of the whole step (four matrices, batch {bsz})")
-        del feeds, vals
-        out[f"batch{bsz}"] = _block(f"C4 decode GEMV, batch {bsz}: x[B,4096] . W_qkv[4096,12288], W_o[4096,4096], "
-                                    "W_gate/up[4096,22016], x[B,11008] . W_down[11008,4096], bf16, one plan",
-                                    "hbm", wbytes, one_us, loop_us, sep_us, info, base)
+        blocks = {}
+        for sets in (2, 1):
+            m = Model()
+            feeds, vals = [], []
+            for rep in range(sets):
+                for name, k, n in shapes:
+                    tx, tw = m.tensor([bsz, k], "bf16"), m.tensor([k, n], "bf16")
+                    m.matmul(tx, tw)
+                    x = inp.normal(f"x_{name}_b{bsz}", tx.shape, torch.bfloat16)
+                    w = inp.normal(name if rep == 0 else f"{name}_set{rep}", tw.shape, torch.bfloat16, 0.02)
+                    feeds += [(tx, x), (tw, w)]
+                    if rep == 0:
+                        vals.append((x, w))
+            plan = m.plan(device_id=0)
+            loop_us, info = _resident_us(torch, Executor, plan, 50, feeds)
+            one_us, sep_us = _oneshot_and_separate_us(torch, Executor, plan, 50, feeds)
+            base = None
+            if cpu and sets == 2:
+                from oracle import ark_oracle as O
+                host = [(x.view(torch.int16).cpu().numpy().view("uint16"), w.view(torch.int16).cpu().numpy().view("uint16"))
+                        for x, w in vals]
+                base = _timed_cpu(lambda: [O.matmul(x, w, "bf16") for x, w in host], wbytes, "GB/s",
+                                  f"oracle matmul of one token step (four matrices, batch {bsz})")
+            del feeds, vals
+            # per token step: a plan iteration is `sets` token steps
+            blocks[sets] = _block(f"C4 decode GEMV, batch {bsz}: x[B,4096] . W_qkv[4096,12288], W_o[4096,4096], "
+                                  "W_gate/up[4096,22016], x[B,11008] . W_down[11008,4096], bf16, one plan; "
+                                  + ("two weight sets in turn (every token step streams from HBM); per token step"
+                                     if sets == 2 else "one weight set, reused every iteration"),
+                                  "hbm", wbytes, one_us / sets, loop_us / sets, sep_us / sets, info, base)
+        blocks[2]["one_weight_set"] = {k: blocks[1][k] for k in ("roofline", "resident_loop_kernel_us", "separate_kernels_us")}
+        out[f"batch{bsz}"] = blocks[2]
     return out
 
 
@@ -459,6 +479,41 @@ def other_configs(torch, np, Model, Executor, llama, prng, cpu, only=None):
     return out
 
 
+def _rows_oneshot_ms(torch, Executor, plan, feeds, steps, launches=10, env=None):
+    """Average duration (ms) of a one-shot launch of `steps` iterations of a row-op plan, under
+    HIP events on the stream the kernel is launched on.  `env` is set while the plan compiles
+    (compile() reads the ARKMI_* switches)."""
+    side = torch.cuda.Stream()
+    old = {k: os.environ.get(k) for k in (env or {})}
+    os.environ.update(env or {})
+    try:
+        ex = Executor(plan, device_id=0, stream=side.cuda_stream, name="bench-oneshot", loop_mode=False).compile()
+    finally:
+        for k, v in old.items():
+            if v is None:
+                del os.environ[k]
+            else:
+                os.environ[k] = v
+    for t, x in feeds:
+        ex.tensor_write_device(t, x)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
+    with torch.cuda.stream(side):
+        ex.launch()
+        ex.run(steps)
+        ex.wait()
+        for s_, e_ in ev:
+            s_.record()
+            ex.run(steps)
+            e_.record()
+        ex.wait()
+    torch.cuda.synchronize()
+    ms = sum(s_.elapsed_time(e_) for s_, e_ in ev) / launches
+    ex.stop()
+    del ex
+    return ms
+
+
 def cpu_baseline_c2(x_np, w_np, min_seconds=8.0):
     """The oracle (a port of the reference's host baselines) timed on this machine's cores:
     passes over one X until `min_seconds` have gone by."""
@@ -564,38 +619,46 @@ def main():
     # ---- roofline of the loop kernel: one-shot launches under HIP events ------------
     # The executor launches on a torch stream (default priority), so torch's events, recorded
     # on that stream, bracket the kernel.
-    side = torch.cuda.Stream()
-    ex1 = Executor(plan, device_id=0, stream=side.cuda_stream, name="bench-oneshot", loop_mode=False).compile()
-    for t, x in zip(tx, xs):
-        ex1.tensor_write_device(t, x)
-    ex1.tensor_write_device(tw, w)
-    torch.cuda.synchronize()
-    launches = 10
-    ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(launches)]
-    with torch.cuda.stream(side):
-        ex1.launch()
-        ex1.run(steps)
-        ex1.wait()
-        for s_, e_ in ev:
-            s_.record()
-            ex1.run(steps)
-            e_.record()
-        ex1.wait()
-    torch.cuda.synchronize()
-    launch_ms = sum(s_.elapsed_time(e_) for s_, e_ in ev) / launches
-    ex1.stop()
-    del ex1
+    feeds = list(zip(tx, xs)) + [(tw, w)]
+    launch_ms = _rows_oneshot_ms(torch, Executor, plan, feeds, steps)
     launch_bytes = step_bytes * steps
     achieved = launch_bytes / (launch_ms * 1e-3) / 1e9
+    # the same plan with every op streaming X from HBM: no byte of the count is a cache hit
+    hbm_ms = _rows_oneshot_ms(torch, Executor, plan, feeds, steps, env={"ARKMI_ROW_CACHED_INPUT": "0"})
+    hbm_only = launch_bytes / (hbm_ms * 1e-3) / 1e9
+    # each op alone over the four rotating X tensors (plans of four ops; nothing is read twice)
+    per_op = {}
+    for name in ("reduce_sum", "softmax", "rmsnorm"):
+        mo = Model()
+        txo = [mo.tensor([ROWS, COLS], "fp16") for _ in range(NBUF)]
+        two = mo.tensor([COLS], "fp32")
+        for t in txo:
+            if name == "reduce_sum":
+                mo.reduce_sum(t, -1)
+            elif name == "softmax":
+                mo.softmax(t)
+            else:
+                mo.rmsnorm(t, two, 1e-6)
+        fo = list(zip(txo, xs)) + ([(two, w)] if name == "rmsnorm" else [])
+        ms = _rows_oneshot_ms(torch, Executor, mo.plan(device_id=0), fo, steps, launches=5)
+        gbps = ALGO_BYTES[name] * NBUF * steps / (ms * 1e-3) / 1e9
+        per_op[name] = {"us_per_X": round(ms * 1e3 / steps / NBUF, 2), "achieved": round(gbps, 1),
+                        "frac": round(gbps / HBM_PEAK_GBPS, 4)}
 
     traffic_per_step, traffic_src = profiled_traffic_bytes_per_step()
     roofline = {"bound": "hbm",
                 "kernel": f"arkmi_loop_kernel<{kernel_families}> (one-shot launch of {steps} plan iterations = steps)",
                 "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                "frac_note": "algorithmic bytes; the second and third read of an X within a step may be served by "
+                             "the Infinity Cache",
+                "achieved_hbm_only": round(hbm_only, 1), "frac_hbm_only": round(hbm_only / HBM_PEAK_GBPS, 4),
+                "hbm_only_note": "the same plan and launch with ARKMI_ROW_CACHED_INPUT=0: every op streams X from HBM",
+                "per_op": per_op,
                 "traffic": traffic_per_step * steps if traffic_per_step else None,
-                "traffic_source": (f"{traffic_src} (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE per step x steps; "
-                                   "not measured in this run)") if traffic_per_step else None,
+                "traffic_source": (f"{traffic_src} (rocprofv3 --pmc FETCH_SIZE + WRITE_SIZE per step x steps: bytes "
+                                   "between the L2s and the fabric, Infinity Cache hits included; not measured in "
+                                   "this run)") if traffic_per_step else None,
                 "launch_ms": round(launch_ms, 4), "launch_algorithmic_bytes": launch_bytes,
                 "us_per_step_in_launch": round(launch_ms * 1e3 / steps, 2)}
 
@@ -605,7 +668,7 @@ def main():
                   "128 MiB, which the Infinity Cache may serve)",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": steps,
         "warmup": warm, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16 (f32 accumulate)",
         "data": "synthetic",
         "config": {"workload": "C2 row ops: X[16384,4096] fp16 ~N(0,1), reduce_sum + softmax + "
                                "RMSNorm(w~U(0.5,1.5), eps=1e-6), fp32 accumulate, one persistent loop "

@@ -132,6 +132,34 @@ def test_matmul_full_size_config(oracle):
     assert float((c2.float() - 2 * c.float()).abs().max()) <= 2.0 ** -22
 
 
+@pytest.mark.parametrize("trans_b", [False, True])
+def test_matmul_full_size_through_the_plan(oracle, trans_b):
+    """The same configuration the way the benchmark runs it: Model -> Planner -> plan -> Executor ->
+    loop kernel (256x256 tiles, the XCD-aware tile order on), two iterations; 256 sampled rows x
+    all columns against the oracle.  With the second operand stored [N, K] too: the layout of every
+    weight matmul in the FFN and the decoder layer."""
+    from ark_amd import Model, Executor, plan_analysis
+    dtype = "fp16"
+    a = make(oracle, (4096, 4096), dtype, seed=21, dist="uniform")
+    b = make(oracle, (4096, 4096), dtype, seed=22, dist="uniform")
+    m = Model()
+    ta, tb = m.tensor([4096, 4096], dtype), m.tensor([4096, 4096], dtype)
+    out = m.matmul(ta, tb, trans_other=trans_b)
+    plan = m.plan(device_id=0)
+    assert plan_analysis(plan)["GemmXcdOrdered"] == 1
+    ex = Executor(plan, device_id=0).compile()
+    ex.tensor_write(ta, a)
+    ex.tensor_write(tb, b)
+    ex.launch()
+    ex.run(2)
+    ex.wait()
+    got = ex.tensor_read(out)
+    ex.stop()
+    rows = np.random.default_rng(1).choice(4096, 256, replace=False)
+    ref = oracle.matmul(np.ascontiguousarray(a[rows]), b, dtype, trans_b=trans_b)
+    _check(oracle, ref, got[rows], dtype, 1.0, 2048)
+
+
 def test_matmul_errors():
     from ark_amd import ops, ArkmiError
     a = torch.zeros(100, 64, dtype=torch.float16, device="cuda")

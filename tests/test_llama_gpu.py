@@ -64,7 +64,7 @@ def test_ffn_small(oracle, dtype):
 def test_ffn_full_size_sampled_rows(oracle, fused):
     """x[8192,4096] bf16 -> 11008 -> 4096 in one loop kernel, as the reference's
     composition and as the fused path the benchmark times (SwiGLU as one GEMM pass);
-    the oracle evaluates 48 sampled rows (every output column of those rows)."""
+    the oracle evaluates 256 sampled rows (every output column of those rows)."""
     from ark_amd import Model, llama
     dtype, rows, dim, hidden = "bf16", 8192, 4096, 11008
     x, w1, w2, w3 = _ffn_case(oracle, rows, dim, hidden, dtype, 200)
@@ -73,7 +73,7 @@ def test_ffn_full_size_sampled_rows(oracle, fused):
     ff = llama.FeedForward(m, dim, hidden, dtype)
     out = ff.forward(tx, fused=fused)
     got, info = _run(m, {tx: x, ff.w1: w1, ff.w2: w2, ff.w3: w3}, out)
-    pick = np.sort(np.random.default_rng(7).choice(rows, 48, replace=False))
+    pick = np.sort(np.random.default_rng(7).choice(rows, 256, replace=False))
     pick[0], pick[-1] = 0, rows - 1
     ref = R.feed_forward(oracle, np.ascontiguousarray(x[pick]), w1, w2, w3, dtype)
     mx, rms = R.composite_error(oracle, ref, got[pick], dtype)
@@ -119,7 +119,7 @@ def test_decoder_layer_small(oracle, dtype, fused):
 @pytest.mark.parametrize("fused", [False, True, "attention", "side_by_side"])
 def test_decoder_layer_full_size_sampled_rows(oracle, fused):
     """Llama-2-7B layer shape: seq 2048, d 4096, 32 heads x 128, SwiGLU 11008,
-    bf16, RoPE base 10000, causal mask.  The oracle evaluates 24 sampled query
+    bf16, RoPE base 10000, causal mask.  The oracle evaluates 256 sampled query
     positions against the whole sequence's keys and values.  "side_by_side": the attention-op
     plan with the query and key projections on 256x256 tiles on the two halves of the processors
     at the same time (no barrier between them)."""
@@ -144,7 +144,7 @@ def test_decoder_layer_full_size_sampled_rows(oracle, fused):
         from ark_amd import plan_schedule
         groups = json.loads(m.plan(device_id=0))["ProcessorGroups"]
         assert [g["ProcessorRange"] for g in groups[1:3]] == [[0, 128], [128, 256]]
-    pick = np.sort(np.random.default_rng(9).choice(seq, 24, replace=False))
+    pick = np.sort(np.random.default_rng(9).choice(seq, 256, replace=False))
     pick[0], pick[-1] = 0, seq - 1
     ref = R.transformer_block(oracle, x, vals, freqs, mask, heads, dtype, q_rows=pick)
     mx, rms = R.composite_error(oracle, ref, got[:, pick], dtype)

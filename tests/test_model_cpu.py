@@ -320,7 +320,7 @@ def test_fused_op_plans_exist_only_on_rocm950():
     plan = json.loads(m.plan(arch="ROCM_950", num_processors=256))
     sw, at = (ti["Ops"][0]["Config"] for ti in plan["TaskInfos"])
     assert sw["TileShapeMNK"] == [256, 256, 64] and sw["NumTasks"] == 8 * 86   # 256 rows x 128 result columns per task
-    assert at["NumTasks"] == 32 * 16 and at["SramBytes"] == 71680              # 128 query positions of one head per task
+    assert at["NumTasks"] == 32 * 16 and at["SramBytes"] == 131072              # 128 query positions of one head per task
     with pytest.raises(ArkmiError) as e:
         m.plan(arch="CUDA_80", num_processors=108)
     assert e.value.kind == "PlanError"
