@@ -78,18 +78,24 @@ class Inputs:
 
 
 def _resident_us(torch, Executor, plan, iters, feeds):
-    """us per iteration in the resident loop kernel (host clock around run() + wait()):
-    `iters` untimed iterations (the clock settles over the first milliseconds of load), then
-    the median of three timed batches."""
+    """us per iteration in the resident loop kernel (host clock around run() + wait()): untimed
+    batches of `iters` iterations for 30 ms, then the median of five timed batches."""
     ex = Executor(plan, device_id=0).compile()
     for t, v in feeds:
         ex.tensor_write_device(t, v)
     torch.cuda.synchronize()
     ex.launch()
+    # untimed load first: the chip leaves its idle clocks over tens of milliseconds, and a batch
+    # timed while they still rise reads up to 10 % slow (one batch here, then as many as 30 ms take)
+    t0 = time.perf_counter()
     ex.run(iters)
     ex.wait()
+    first = time.perf_counter() - t0
+    for _ in range(min(50, int(0.03 / max(first, 1e-6)))):
+        ex.run(iters)
+        ex.wait()
     batches = []
-    for _ in range(3):
+    for _ in range(5):
         t0 = time.perf_counter()
         ex.run(iters)
         ex.wait()
@@ -97,7 +103,7 @@ def _resident_us(torch, Executor, plan, iters, feeds):
     info = ex.info()
     ex.stop()
     del ex
-    return sorted(batches)[1], info
+    return sorted(batches)[2], info
 
 
 def _oneshot_and_separate_us(torch, Executor, plan, iters, feeds):
@@ -592,6 +598,10 @@ def main():
     torch.cuda.synchronize()
 
     steps, warm = max(1, args.steps), max(0, args.warmup)
+    # The machine probes (a few hundred milliseconds of MFMA and streaming load) run first: the
+    # chip leaves its idle clocks over tens of milliseconds of load, longer than the warm-up steps
+    # last, and the timed steps should see the clocks every later measurement of this run sees.
+    machine = machine_probes(torch, prng)
     # The loop kernel stays resident between run() calls, so a device-wide synchronize inside
     # the timed region would wait for it to leave; Executor.wait() is the completion point.
     ex.launch()
@@ -675,7 +685,7 @@ def main():
                                "kernel; a step = the three ops over each of 4 rotating X tensors",
                    "device": info["gcn_arch"], "num_cu": info["num_cu"]},
         "roofline": roofline,
-        "machine": machine_probes(torch, prng),
+        "machine": machine,
     }
     if not args.no_extra:
         out["configs"] = other_configs(torch, np, Model, Executor, llama, prng, cpu)
