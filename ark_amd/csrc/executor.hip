@@ -675,6 +675,15 @@ DevOp lower_op(const Json &op_json, const Lowering &L, int slot_warps, int block
         w.op = e.op;
         if (e.op == EW_SCALAR_ASSIGN) w.param = f_arg("Value");
         if (e.op == EW_SCALAR_ADD || e.op == EW_SCALAR_MUL) w.param = f_arg("Factor");
+        if (w.dt_out == 3 && (e.op == EW_SCALAR_ASSIGN || e.op == EW_SCALAR_ADD || e.op == EW_SCALAR_MUL)) {
+            // The scalar travels as a float (as in the plan file) and the body
+            // converts it to int32 by truncation.  That conversion is defined
+            // only inside the int32 range; a value beyond 2^24 in magnitude is
+            // already rounded to float precision when it gets here.
+            const float v = w.param;
+            if (!(v >= -2147483648.0f && v < 2147483648.0f))
+                ARK_ERR(UnsupportedError, "op ", type, ": INT32 scalar ", v, " is outside the int32 range");
+        }
         if (!cfg.contains("Tile")) ARK_ERR(PlanError, type, " config needs Tile");
         auto tile = cfg.at("Tile").as_int_vector();
         int64_t th = tile.at(0), tw = tile.at(1);

@@ -7,8 +7,9 @@ libarkmi.so; nothing here computes.
 """
 import ctypes
 import json
+import math
 
-from ._lib import lib, check, DTYPES
+from ._lib import lib, check, DTYPES, InvalidUsageError
 
 _DT_NAMES = {v: k for k, v in DTYPES.items()}
 
@@ -136,6 +137,10 @@ class Model:
         res = (ctypes.c_int64 * 64)()
         n = ctypes.c_int()
         args = {k: v for k, v in args.items() if v is not None}
+        for k, v in args.items():
+            # a plan file is JSON, which has no spelling for inf or nan
+            if isinstance(v, float) and not math.isfinite(v):
+                raise InvalidUsageError(f"op {op}: argument {k} = {v} is not finite")
         check(lib().arkmi_model_op(self._h, op.encode(), _i64(ins), ctypes.c_int(len(ins)),
                                    ctypes.c_int64(output.id if output is not None else -1),
                                    json.dumps(args).encode(), name.encode(), res, ctypes.c_int(64),

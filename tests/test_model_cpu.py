@@ -345,3 +345,32 @@ def test_embedding_shapes_and_invalid():
     p = json.loads(m.plan(arch="ROCM_950", num_processors=256))
     cfg = p["TaskInfos"][0]["Ops"][0]["Config"]
     assert cfg["NumWarps"] == 8 and cfg["NumTasks"] == 8 * 3 * 64 // 8
+
+
+def test_int32_scalars_outside_the_int32_range_are_refused():
+    """A scalar operand travels as a float, in the plan file and to the kernel
+    (ark/ops/ops_scalar.cpp:82-111 keeps "Factor" as a float too), and the INT32 body
+    truncates it to the element type like ark/include/kernels/scalar.h:13-41.  That
+    conversion is defined inside the int32 range only: compile() refuses the rest, and
+    a scalar that JSON cannot spell is refused when the op is made."""
+    from ark_amd import Model, plan_analysis, ArkmiError
+
+    def compile_with(v):
+        m = Model()
+        t = m.tensor([64, 256], "int32")
+        m.mul(t, v)
+        plan_analysis(m.plan(arch="ROCM_950", num_processors=256), 0)
+
+    for v in (0.0, 3.5, -7.9, 16777218.0, 2147483520.0, -2147483648.0):
+        compile_with(v)
+    for v in (2147483648.0, 3e9, -2147483904.0, -3e9, 1e30):
+        with pytest.raises(ArkmiError) as e:
+            compile_with(v)
+        assert e.value.kind == "UnsupportedError" and "INT32 scalar" in str(e.value)
+    for v in (float("inf"), float("nan")):
+        with pytest.raises(ArkmiError) as e:
+            compile_with(v)
+        assert e.value.kind == "InvalidUsageError" and "not finite" in str(e.value)
+    m = Model()
+    m.mul(m.tensor([64, 256], "fp32"), 1e30)   # float tensors take any finite scalar
+    plan_analysis(m.plan(arch="ROCM_950", num_processors=256), 0)
