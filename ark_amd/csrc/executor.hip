@@ -428,12 +428,24 @@ DevOp lower_op(const Json &op_json, const Lowering &L, int slot_warps, int block
             ARK_ERR(PlanError, "Matmul: NumTasks must be SplitK * batch * (M / ", tm, ") * (N / ", tn, ") = ",
                     tiles * g.split_k, ", got ", cfg.at("NumTasks").as_int());
         if (g.split_k == 2) {
-            if (tm != 256 || tn != 256 || ta || f32 || (g.k % (4 * kGemmMinK / 2)))
+            if (tm != 256 || tn != 256 || ta || f32 || (g.k % (2 * kGemmMinK)) || g.k < 8 * kGemmMinK)
                 ARK_ERR(UnsupportedError, "Matmul: SplitK 2 runs on 256x256 tiles of FP16/BF16 operands with K % ",
-                        2 * kGemmMinK, " == 0 and no TransposeInput");
-            // partial accumulators of both halves + one arrival counter per tile
+                        2 * kGemmMinK, " == 0, K >= ", 8 * kGemmMinK, " and no TransposeInput");
+            // The sender's part of K is shorter by twice the skew: its partial sums are then
+            // written while the finisher still multiplies, and the finisher finds them there.
+            // (2048 x 4096 x 4096, finisher's time: 70.6 us with equal parts, 67.5 with 192, 72.2
+            // with 384; writing and announcing a tile's partial sums takes the time of ~6 K tiles.)
+            int64_t skew = 192;
+            if (const char *e = std::getenv("ARKMI_SPLITK_SKEW")) skew = std::atoll(e);
+            skew = std::max<int64_t>(0, skew) / kGemmMinK * kGemmMinK;
+            const int64_t min_part = 4 * kGemmMinK;  // a part of K fills the stage ring at least once
+            int64_t at = (int64_t)g.k / 2 + skew;
+            at = std::min<int64_t>(at, g.k - min_part);
+            at = std::max<int64_t>(at, min_part);
+            g.split_at = (int)at;
+            // the sender's partial accumulators + one full/empty word per tile
             const size_t counter_bytes = ((size_t)tiles * 4 + 255) / 256 * 256;
-            const size_t tile_bytes = (size_t)2 * kGemmThreads * (256 / 2 / 16) * (256 / 4 / 16) * 16;
+            const size_t tile_bytes = (size_t)kGemmThreads * (256 / 2 / 16) * (256 / 4 / 16) * 16;
             char *ws = static_cast<char *>(L.scratch(counter_bytes + (size_t)tiles * tile_bytes));
             g.arrivals = reinterpret_cast<unsigned int *>(ws);
             g.partial = reinterpret_cast<float *>(ws + counter_bytes);
@@ -726,6 +738,55 @@ DevOp lower_op(const Json &op_json, const Lowering &L, int slot_warps, int block
 // data hazards between task groups (for eliding barriers nobody needs)
 // ---------------------------------------------------------------------------
 namespace {
+
+// A matmul with one elementwise op behind it (Add, Sub, Mul, Div with the matmul's result as
+// either input; Rope with it as the first): where every tile of C leaves through the staged
+// store of gemm_tile and the op's operands are dense rows aligned to 16 bytes, the op is
+// folded into that store (GemmDesc::fuse_*) instead of reading the tile back.  The values are
+// the same bits either way: the store rounds C to the tensor type first, as the op would read
+// it.  ARKMI_GEMM_FOLD_STORE=0 keeps the op a pass of its own.
+static bool fold_into_store(DevOp &lead, const DevOp &next) {
+    if (const char *e = getenv("ARKMI_GEMM_FOLD_STORE"))
+        if (atoi(e) == 0) return false;
+    if (lead.kind != DEV_GEMM || next.kind != DEV_EWISE) return false;
+    GemmDesc &g = lead.gemm;
+    const EwiseDesc &w = next.ew;
+    const int tm = lead.gemm_tile_m, tn = lead.gemm_tile_n;
+    // the staged store: fp16/bf16 tiles 128 or 256 columns wide, whole tiles, aligned rows
+    if ((g.dtype != 1 && g.dtype != 2) || g.trans_a || g.b2 || g.batch_total != 1) return false;
+    if ((tn != 128 && tn != 256) || (tm != 128 && tm != 256)) return false;
+    if (g.store_m % tm || g.store_n % tn || (g.ldc % 8) || ((uintptr_t)g.c % 16)) return false;
+    const bool arith = w.op == EW_ADD || w.op == EW_SUB || w.op == EW_MUL || w.op == EW_DIV;
+    if (!arith && w.op != EW_ROPE) return false;
+    if (w.dt_in != g.dtype || w.dt_out != g.dtype || !w.fast) return false;
+    if (w.shape[0] != 1 || w.shape[1] != 1 || w.shape[2] != g.store_m || w.shape[3] != g.store_n) return false;
+    if (w.tile_h != tm || w.tile_w != tn) return false;
+    auto is_c = [&](const EwTensor &t) { return t.ptr == g.c && t.s[2] == g.ldc && t.s[3] == 1; };
+    auto dense_rows = [](const EwTensor &t) {
+        return t.s[3] == 1 && ((uintptr_t)t.ptr % 16) == 0 && (t.s[2] % 8) == 0 && t.s[2] >= 0 &&
+               t.s[2] < ((int64_t)1 << 31);
+    };
+    const EwTensor *other = nullptr;
+    int c_second = 0, period = 0;
+    if (is_c(w.in0)) {
+        other = &w.in1;
+        period = w.in1_period;
+    } else if (arith && is_c(w.in1) && w.in1_period == 0) {
+        other = &w.in0;
+        c_second = 1;
+    } else {
+        return false;
+    }
+    if (!dense_rows(*other) || !dense_rows(w.out) || w.out.s[2] == 0 || period < 0 || (period % 8)) return false;
+    g.fuse_other = other->ptr;
+    g.fuse_out = w.out.ptr;
+    g.fuse_kind = 1 + w.op;
+    g.fuse_c_second = c_second;
+    g.fuse_ld_other = (int)other->s[2];
+    g.fuse_ld_out = (int)w.out.s[2];
+    g.fuse_period = period;
+    return true;
+}
 
 struct Access {
     size_t buffer;
@@ -1154,6 +1215,7 @@ struct Executor {
     int kernel_families = 0;      // the loop-kernel variant in use
     const void *kernel = nullptr;
     std::vector<void *> scratch_allocs;  // per-op device scratch (split-K partials, counters)
+    std::vector<char> group_fused;       // per task group: its elementwise follower rides in the matmul's store
     std::vector<int> h_group_fam;        // OpFamily bits of each task group
     std::vector<const void *> step_kernels_ready;  // step kernels whose LDS limit is set
     std::vector<int> dev_step_of;  // schedule step -> device step, -1 if elided
@@ -1265,9 +1327,11 @@ struct Executor {
         std::vector<DevOp> ops;
         std::vector<DevStep> steps;
         h_groups.clear();
+        group_fused.clear();
         h_group_fam.clear();
         group_sched_step.clear();
         int max_slot_lds = 0;
+        int n_split_matmuls = 0;
         trace_len = 0;
         const Json &task_infos = plan.at("TaskInfos");
         // A barrier of the reference's schedule orders *processors*, whether
@@ -1401,6 +1465,21 @@ struct Executor {
                                     "behind a matmul");
                     }
                 }
+                if (ops[(size_t)g.op_begin].kind == DEV_GEMM && ops[(size_t)g.op_begin].gemm.split_k == 2) {
+                    // Split matmuls alternate which half of their tasks sends and which finishes:
+                    // a finisher works ~10 us longer than its sender, and with the same
+                    // workgroups finishing every time (Q, K, V projections in a row, no barrier
+                    // between them) the others would idle for the sum.  Only where a workgroup
+                    // runs at most one task of the matmul (see GemmDesc::split_flip).
+                    const char *env = getenv("ARKMI_SPLITK_ALTERNATE");
+                    const int n_tasks = (st.task_e - st.task_b + st.task_s - 1) / st.task_s;
+                    const int n_procs = (st.proc_e - st.proc_b + st.proc_s - 1) / st.proc_s;
+                    if (env && atoi(env) == 1 && st.n_slots == 1 && n_tasks <= n_procs)
+                        ops[(size_t)g.op_begin].gemm.split_flip = n_split_matmuls & 1;
+                    ++n_split_matmuls;
+                }
+                group_fused.push_back(g.op_count == 2 && fold_into_store(ops[(size_t)g.op_begin],
+                                                                          ops[(size_t)g.op_begin + 1]) ? 1 : 0);
                 int group_fam = 0;
                 for (int o = g.op_begin; o < (int)ops.size(); ++o)
                     group_fam |= ops[o].kind == DEV_ROW ? (ops[o].row.red_len > 0 ? FAM_EXT : FAM_ROW)
@@ -1943,7 +2022,13 @@ struct Executor {
             if (bytes) ARKMI_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
         };
         upload(ops.data(), ops.size() * sizeof(DevOp), (void **)&d_ops);
-        upload(h_groups.data(), h_groups.size() * sizeof(DevTaskGroup), (void **)&d_groups);
+        {
+            // a follower folded into its matmul's store does not run as an op of its own
+            std::vector<DevTaskGroup> dev_groups = h_groups;
+            for (size_t gi = 0; gi < dev_groups.size(); ++gi)
+                if (group_fused[gi]) dev_groups[gi].op_count = 1;
+            upload(dev_groups.data(), dev_groups.size() * sizeof(DevTaskGroup), (void **)&d_groups);
+        }
         upload(steps.data(), steps.size() * sizeof(DevStep), (void **)&d_steps);
         if (trace_enabled && trace_len) {
             ARKMI_HIP(hipMalloc((void **)&d_trace, trace_len * sizeof(TraceRecord)));
@@ -2057,6 +2142,8 @@ struct Executor {
         if (!compiled) ARK_ERR(InvalidUsageError, "Need to compile first.");
         if (launched && loop_mode) ARK_ERR(InvalidUsageError, "stop the loop kernel before running its ops as separate kernels");
         set_device();
+        // the bodies' bounded waits (the split of K) use the control block's abort word
+        ARKMI_HIP(hipMemsetAsync(ctl, 0, sizeof(LoopControl), stream));
         for (int it = 0; it < iter; ++it) {
             for (size_t gi = 0; gi < h_groups.size(); ++gi) {
                 const void *k = step_kernel_select(h_group_fam[gi]);
@@ -2065,8 +2152,8 @@ struct Executor {
                     step_kernels_ready.push_back(k);
                 }
                 const DevTaskGroup &g = h_groups[gi];
-                step_kernel_launch(k, prog, (int)gi, grid, threads,
-                                   loop_kernel_lds_reserved() + g.n_slots * g.slot_sram, stream);
+                step_kernel_launch(k, prog, ctl, mb_dev, (int)gi, grid, threads,
+                                   loop_kernel_lds_reserved() + g.n_slots * g.slot_sram, wait_ticks, stream);
             }
         }
     }
@@ -2516,8 +2603,13 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
                 if (ex.dry_ops.size() > (size_t)g.op_begin && ex.dry_ops[(size_t)g.op_begin].kind == arkmi::DEV_GEMM) {
                     j["XcdRound"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.xcd_round;
                     j["XcdBand"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.xcd_band;
+                    if (ex.dry_ops[(size_t)g.op_begin].gemm.split_k == 2) {
+                        j["SplitAt"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.split_at;
+                        j["SplitFlip"] = ex.dry_ops[(size_t)g.op_begin].gemm.split_flip != 0;
+                    }
                 }
                 j["Claimed"] = g.claim >= 0;
+                j["FoldedIntoStore"] = (size_t)st.index < ex.group_fused.size() && ex.group_fused[(size_t)st.index] != 0;
                 Json waits = Json::array();
                 for (int w = 0; w < g.n_waits; ++w) {
                     const arkmi::DevWait &dw = ex.dry_waits[(size_t)(g.wait_begin + w)];

@@ -169,11 +169,12 @@ static Json rocm950_config(const ModelOp &op, int num_cu) {
                     " should be divisible by a tile shape of 128x128x64 or larger");
         // An output that gives 256x256 tiles to between half and all of the CUs, with a long K:
         // keep the large tile (two thirds of the operand traffic per flop of a 128x256 tile) and
-        // split K in two, so the tiles' halves fill the chip; the half that finishes second adds
-        // the two.  The exchange of partial sums costs about 16 us, which a 128x256 tiling loses
-        // only from K = 8192 on (2048 x 4096 x 11008: 163 against 185 us; x 4096: 78 either way).
+        // split K in two, so the tiles' halves fill the chip: one task sends its partial sums,
+        // the other adds them to its own and finishes the tile.  The exchange costs the finisher
+        // about 9 us, which a 256x128 tiling loses from K = 4096 on (2048 x 4096 x 4096: 69
+        // against 75 us; x 11008: 154 against 185 us).
         int64_t split = 1;
-        if (!trans_in && !f32 && mnk[0] % 256 == 0 && mnk[1] % 256 == 0 && mnk[2] % 128 == 0 && mnk[2] >= 8192) {
+        if (!trans_in && !f32 && mnk[0] % 256 == 0 && mnk[1] % 256 == 0 && mnk[2] % 128 == 0 && mnk[2] >= 4096) {
             const int64_t tiles256 = batch * (mnk[0] / 256) * (mnk[1] / 256);
             if (tiles256 < num_cu && 2 * tiles256 >= num_cu) {
                 tm = tn = 256;

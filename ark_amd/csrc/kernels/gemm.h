@@ -27,6 +27,9 @@
 // Tile index semantics follow ark/include/kernels/common/unit_op.h:73-92:
 // task -> (batch, m_tile, n_tile) row-major with the N tile fastest.
 #pragma once
+#include <type_traits>
+
+#include "ewise.h"
 #include "dev_common.h"
 
 namespace arkmi {
@@ -51,16 +54,89 @@ struct GemmDesc {
     int32_t dtype;             // 1 fp16, 2 bf16; 0 fp32 (kernels/gemm_f32.h, 128x128 tiles)
     int32_t tiles_m, tiles_n;  // ceil(m/BM), ceil(n/BN)
     int32_t store_m, store_n;  // rows/cols of C that exist (unpadded shape)
-    // Two-way split of K (split_k == 2): task t and task t + tiles each multiply half of K for
-    // tile t; both leave their fp32 accumulators in `partial` and count in `arrivals[t]`; the one
-    // that arrives second adds the other's and finishes the tile.  Nobody waits.
+    // Two-way split of K (split_k == 2): task t multiplies K from split_at on for tile t and
+    // leaves its fp32 accumulators in `partial`; task t + tiles multiplies K below split_at,
+    // adds those and finishes the tile.  `arrivals[t]` is the full/empty word of the tile's
+    // partial sums: 0 empty (the sender may write), 1 full (the finisher may read).  The
+    // sender's part of K is the shorter one, so that its partial sums are on their way while
+    // the finisher still multiplies.
     int32_t split_k;           // 1 or 2
     // XCD-aware order of the tiles (gemm_tile): xcd_round > 0 turns it on
     int32_t xcd_round, xcd_band;
-    int32_t pad_;
-    float *partial;            // [tiles][2 halves][MT * NT][512 threads] x 4 floats
-    unsigned int *arrivals;    // [tiles], zero between uses
+    int32_t split_at;          // split_k == 2: where the sender's part of K begins
+    float *partial;            // [tiles][MT * NT][512 threads] x 4 floats
+    unsigned int *arrivals;    // [tiles], zero between launches
+    // An elementwise op folded into the store of C (fuse_kind != 0; the host sets it only where
+    // every tile takes the staged store of gemm_tile): the values of C, rounded to the tensor
+    // type as they are stored, meet the op's other operand, 16 bytes per lane, and the result
+    // goes to fuse_out.  C itself is stored as always.
+    const void *fuse_other;
+    void *fuse_out;
+    int32_t fuse_kind;         // 0: none; else 1 + EwOp (EW_ADD, EW_SUB, EW_MUL, EW_DIV, EW_ROPE)
+    int32_t fuse_c_second;     // 1: C is the op's second input and the other operand its first
+    int32_t fuse_ld_other;     // elements between rows of the other operand (0: one row for all)
+    int32_t fuse_ld_out;       // elements between rows of the result
+    int32_t fuse_period;       // > 0: the other operand's column is taken modulo this (a multiple of 8)
+    // split_k == 2: 1 swaps the roles, tasks [0, tiles) finish and tasks [tiles, 2 tiles) send (set
+    // only where a workgroup runs one task of the matmul: a finisher must never stand in front of
+    // a sender on the same workgroup)
+    int32_t split_flip;
 };
+
+// Eight values of C (as stored) and eight of the other operand through elementwise op `op`,
+// with the arithmetic and the roundings of the op's own body (ew_compute).
+template <typename T>
+__device__ __forceinline__ uint32_t __attribute__((ext_vector_type(4)))
+fused_store_values(int op, bool c_second, uint32_t __attribute__((ext_vector_type(4))) cv,
+                   uint32_t __attribute__((ext_vector_type(4))) ov) {
+    T c[kEwGroup], o[kEwGroup], r[kEwGroup];
+    __builtin_memcpy(c, &cv, 16);
+    __builtin_memcpy(o, &ov, 16);
+    float a[kEwGroup], b[kEwGroup], y[kEwGroup];
+#pragma unroll
+    for (int j = 0; j < kEwGroup; ++j) {
+        const float fc = ew_to_f32<T>(c[j]), fo = ew_to_f32<T>(o[j]);
+        a[j] = c_second ? fo : fc;
+        b[j] = c_second ? fc : fo;
+    }
+    switch (op) {
+        case EW_ADD: ew_compute<T, EW_ADD>(a, b, 0.f, y); break;
+        case EW_SUB: ew_compute<T, EW_SUB>(a, b, 0.f, y); break;
+        case EW_MUL: ew_compute<T, EW_MUL>(a, b, 0.f, y); break;
+        case EW_DIV: ew_compute<T, EW_DIV>(a, b, 0.f, y); break;
+        default: ew_compute<T, EW_ROPE>(a, b, 0.f, y); break;
+    }
+#pragma unroll
+    for (int j = 0; j < kEwGroup; ++j) r[j] = ew_from_f32<T>(y[j]);
+    uint32_t __attribute__((ext_vector_type(4))) out;
+    __builtin_memcpy(&out, r, 16);
+    return out;
+}
+
+// What a bounded wait inside a body needs: the kernel's abort word and the tick limit.
+struct BodyWait {
+    int32_t *abort;
+    uint64_t limit_ticks;
+};
+constexpr int kGemmAborted = -3;  // gemm_tile: a bounded wait gave up (the kernel's abort word is set)
+
+// Polls *word until it reads `want`; false once the abort word is set or the limit has passed
+// (then the abort word is set for everyone).
+__device__ __forceinline__ bool poll_equals(unsigned int *word, unsigned int want, const BodyWait &w) {
+    const uint64_t t0 = wall_clock64();
+    unsigned polls = 0;
+    while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want) {
+        __builtin_amdgcn_s_sleep(1);
+        if ((++polls & 63u) == 0) {
+            if (__hip_atomic_load(w.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
+            if (wall_clock64() - t0 > w.limit_ticks) {
+                __hip_atomic_store(w.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return false;
+            }
+        }
+    }
+    return true;
+}
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
@@ -127,20 +203,29 @@ struct EpilogueStore {
 };
 
 // Returns the tile this workgroup finished (its followers — the elementwise ops fused behind the
-// matmul — run for that tile index), or -1 when the other half of a split tile will finish it.
+// matmul — run for that tile index), -1 when the other half of a split tile will finish it, or
+// kGemmAborted.
+// `poll(word, want)` is the bounded wait of the split (poll_equals with the kernel's abort word
+// and tick limit, which the caller reads where it waits rather than carry them through the K loop).
+struct NoPoll {
+    __device__ __forceinline__ bool operator()(unsigned int *, unsigned int) const { return true; }
+};
 template <typename T, int BM, int BN, bool TRANS_B, typename Epi, bool TRANS_A = false, bool DUAL_B = false,
-          bool SPLIT = false>
-__device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const Slot &s, Epi epi) {
+          bool SPLIT = false, typename Poll = NoPoll>
+__device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const Slot &s, Epi epi, Poll poll = Poll()) {
+    static_assert(!SPLIT || !std::is_same<Poll, NoPoll>::value, "the split of K needs a bounded wait");
     static_assert(!DUAL_B || (TRANS_B && !TRANS_A), "the gate/up pair takes K-contiguous operands");
     static_assert(!SPLIT || (!DUAL_B && !TRANS_A), "the split of K exists for plain matmuls");
-    // split: tasks [0, tiles) take the upper half of K, tasks [tiles, 2 tiles) the lower half
+    // split: tasks [0, tiles) send the part of K from split_at on, tasks [tiles, 2 tiles) multiply
+    // the part below it and finish the tile.  A workgroup runs its tasks in rising order, so a
+    // sender never stands behind a finisher that waits for it.  (split_flip swaps the two roles.)
     int task = task_in, k_begin = 0, k_len = d.k, half = 0;
     if constexpr (SPLIT) {
         const int tiles = d.tiles_m * d.tiles_n * d.batch_total;
-        half = task_in >= tiles ? 0 : 1;
+        half = (task_in >= tiles ? 0 : 1) ^ (d.split_flip ? 1 : 0);
         task = task_in >= tiles ? task_in - tiles : task_in;
-        k_len = d.k / 2;
-        k_begin = half * k_len;
+        k_begin = half ? d.split_at : 0;
+        k_len = half ? d.k - d.split_at : d.split_at;
     }
     constexpr int BK = GemmShape<BM, BN>::BK;
     constexpr int S = GemmShape<BM, BN>::STAGES;
@@ -485,50 +570,118 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     // buffers are used again (by the next task or another op body)
     wait_vmcnt_then_barrier<0>();
 
+    // The wave's output: NTO column tiles of 16 per 16-row strip.  For the gate/up pair accumulator
+    // tiles j and j + NT/2 of a wave hold the gate and the up product of the same 16 output columns.
+    static_assert(!DUAL_B || NT % 2 == 0, "the gate/up pair needs an even number of column tiles per wave");
+    constexpr int NTO = DUAL_B ? NT / 2 : NT;
+    const int col_w = DUAL_B ? tn * (BN / 2) + wn * (WTN / 2) : n0 + wn * WTN;  // the wave's first output column
+    const int out_n0 = DUAL_B ? tn * (BN / 2) : n0, out_bn = DUAL_B ? BN / 2 : BN;
+    // Whole tiles of an aligned C go through LDS, strip by strip: a wave writes a strip of 16 rows
+    // x (16 NTO) columns (8 bytes per lane and column tile) into a window of its own and reads it
+    // back as 16 bytes per lane, LPR lanes to a row: every store instruction then writes whole row
+    // segments (128 bytes, a cache line, for four column tiles), where the accumulator layout by
+    // itself gives 32 bytes per row and instruction and the L2 writes some lines back more than
+    // once.  No barrier inside: a wave's LDS operations complete in order and the window is the
+    // wave's own (the stage ring is free: the K loop ended with every load landed and every wave
+    // past its last fragment read).
+    constexpr int SEG_B = NTO * 16 * 2;           // bytes of a strip's row
+    constexpr int SPITCH = SEG_B + 16;            // padded: rows 16 bytes apart modulo the bank span
+    constexpr int LPR = SEG_B / 16;               // lanes per row when reading back
+    constexpr int RPP = 64 / LPR;                 // rows per pass
+    constexpr bool kStaged = (64 % LPR == 0) && (RPP <= 16) && (16 % RPP == 0);
+    // An elementwise op folded into the store (fuse_kind): the other operand's segments of the whole
+    // tile are requested ahead of the strips, which take a fraction of a memory round trip each
+    // (fetched one strip ahead, every strip waited for its segment): all of them here; for a
+    // split tile the first quarter here, before the finisher waits for and adds the sender's
+    // partial sums, and the rest after (the registers do not hold both at once).
+    constexpr int PASSES = kStaged ? 16 / RPP : 1;
+    const int rrow = lane / LPR, rchunk = lane % LPR;
+    const bool fuse = !DUAL_B && kStaged && d.fuse_kind != 0 && (!SPLIT || half == 0);
+    u32x4 oth[MT][PASSES];
+    gptr<const T> other = as_global(static_cast<const T *>(d.fuse_other));
+    gptr<T> fout = as_global(static_cast<T *>(d.fuse_out));
+    int ocol = col_w + rchunk * 8;
+    if (fuse && d.fuse_period > 0) ocol %= d.fuse_period;
+    auto other_load = [&](int i, u32x4(&dst)[PASSES]) {
+#pragma unroll
+        for (int p = 0; p < PASSES; ++p) {
+            const int row = m0 + wm * WTM + i * 16 + p * RPP + rrow;
+            dst[p] = *(const ARKMI_GLOBAL u32x4 *)(other + (int64_t)row * d.fuse_ld_other + ocol);
+        }
+    };
+    constexpr int FIRST = SPLIT ? (MT + 3) / 4 : MT;
+    if (fuse) {
+#pragma unroll
+        for (int i = 0; i < FIRST; ++i) other_load(i, oth[i]);
+    }
+
     if constexpr (SPLIT) {
-        // Partials travel as agent-scope relaxed atomics (write-through stores, L2-bypassing
-        // loads): the two halves run on different XCDs, whose L2s do not see each other.
-        // Ordering: every wave waits for its stores to be acknowledged before the workgroup
-        // barrier, the arrival is counted after it, and the other half's partials are read only
-        // by the workgroup that saw the count at one.
-        // 16-byte buffer stores and loads with the agent-scope bit (sc1): written through to
-        // memory and read past this XCD's L2, at full width (8-byte atomics write half lines).
+        // The partial sums cross from one XCD to another, whose L2s do not see each other:
+        // 16-byte buffer stores and loads with the agent-scope bit (sc1), written through to
+        // memory and read past this XCD's L2.  Ordering: every wave of the sender waits for its
+        // stores to be acknowledged before the workgroup barrier, the word is set to full after
+        // it; the finisher reads only after it has seen full, and sets empty only after its
+        // last load has returned.
         constexpr int PER_THREAD = MT * NT;  // f32x4 values
         constexpr int kAgentScope = 16;      // cache-policy bit sc1 of the buffer instructions
-        const int64_t tile_bytes = (int64_t)2 * kGemmThreads * PER_THREAD * 16;
+        const int64_t tile_bytes = (int64_t)kGemmThreads * PER_THREAD * 16;
         char *tile_base = reinterpret_cast<char *>(d.partial) + (int64_t)task * tile_bytes;
         const __amdgpu_buffer_rsrc_t rsrc =
             __builtin_amdgcn_make_buffer_rsrc(tile_base, 0, (int)tile_bytes, 0x00020000);
-        // [half][row tile * NT + column tile][thread]: a wave's store covers 1 KB in one piece
-        const int mine = (half * PER_THREAD * kGemmThreads + tid) * 16;
-        const int theirs = ((half ^ 1) * PER_THREAD * kGemmThreads + tid) * 16;
+        // [row tile * NT + column tile][thread]: a wave's store covers 1 KB in one piece
+        const int at = tid * 16;
+        unsigned int *word = d.arrivals + task;
+        lds_i32x *verdict = (lds_i32x *)lds;
+        if (tid == 0) *verdict = poll(word, half ? 0u : 1u) ? 1 : 0;
+        s.sync();
+        const bool go = *verdict != 0;
+        s.sync();  // the verdict word is part of the stage buffers the next task refills
+        if (!go) return kGemmAborted;
+        if (half) {
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
+            for (int i = 0; i < MT; ++i) {
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rsrc,
+                                                           at + (i * NT + j) * kGemmThreads * 16, 0, kAgentScope);
+                __builtin_amdgcn_sched_barrier(0);  // row tile by row tile: no pile of addresses and values
+            }
+            drain_stores_then_barrier();
+            if (tid == 0) __hip_atomic_store(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return -1;
+        }
+        // the finisher: AHEAD row tiles of loads in flight while one is added
+#ifndef ARKMI_SPLIT_AHEAD
+#define ARKMI_SPLIT_AHEAD 4
+#endif
+        constexpr int AHEAD = MT < ARKMI_SPLIT_AHEAD ? MT : ARKMI_SPLIT_AHEAD;
+        u32x4 in[AHEAD][NT];
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i)
 #pragma unroll
             for (int j = 0; j < NT; ++j)
-                __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, acc[i][j]), rsrc,
-                                                       mine + (i * NT + j) * kGemmThreads * 16, 0, kAgentScope);
-            __builtin_amdgcn_sched_barrier(0);  // row tile by row tile: no pile of addresses and values
-        }
-        drain_stores_then_barrier();
-        lds_i32x *flag = (lds_i32x *)lds;
-        if (tid == 0)
-            *flag = (int)__hip_atomic_fetch_add(d.arrivals + task, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s.sync();
-        const int arrived_before = *flag;
-        s.sync();  // the flag word is part of the stage buffers the next task refills
-        if (arrived_before == 0) return -1;
-        if (tid == 0) __hip_atomic_store(d.arrivals + task, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                in[i][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, at + (i * NT + j) * kGemmThreads * 16, 0,
+                                                                 kAgentScope);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
 #pragma unroll
-            for (int j = 0; j < NT; ++j) {
-                const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(
-                    rsrc, theirs + (i * NT + j) * kGemmThreads * 16, 0, kAgentScope);
-                acc[i][j] += __builtin_bit_cast(f32x4, w);
+            for (int j = 0; j < NT; ++j) acc[i][j] += __builtin_bit_cast(f32x4, in[i % AHEAD][j]);
+            if (i + AHEAD < MT) {
+#pragma unroll
+                for (int j = 0; j < NT; ++j)
+                    in[i % AHEAD][j] = __builtin_amdgcn_raw_buffer_load_b128(
+                        rsrc, at + ((i + AHEAD) * NT + j) * kGemmThreads * 16, 0, kAgentScope);
             }
-            __builtin_amdgcn_sched_barrier(0);  // a row tile's loads in flight at a time
+            __builtin_amdgcn_sched_barrier(0);
         }
+        wait_vmcnt_then_barrier<0>();
+        if (tid == 0) __hip_atomic_store(word, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+
+    if (fuse) {
+#pragma unroll
+        for (int i = FIRST; i < MT; ++i) other_load(i, oth[i]);
     }
 
     // ---- epilogue: lane (m = lane%16, g = lane/16) holds C[m][4g .. 4g+3] of each 16x16 tile ----
@@ -550,12 +703,6 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
                 if (col + e < d.store_n) p[e] = from_f32<T>(v[e]);
         }
     };
-    // The wave's output: NTO column tiles of 16 per 16-row strip.  For the gate/up pair accumulator
-    // tiles j and j + NT/2 of a wave hold the gate and the up product of the same 16 output columns.
-    static_assert(!DUAL_B || NT % 2 == 0, "the gate/up pair needs an even number of column tiles per wave");
-    constexpr int NTO = DUAL_B ? NT / 2 : NT;
-    const int col_w = DUAL_B ? tn * (BN / 2) + wn * (WTN / 2) : n0 + wn * WTN;  // the wave's first output column
-    const int out_n0 = DUAL_B ? tn * (BN / 2) : n0, out_bn = DUAL_B ? BN / 2 : BN;
     auto value4 = [&](int i, int j, int row, int col, float *o) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -567,23 +714,9 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
             }
         }
     };
-    // Whole tiles of an aligned C go through LDS, strip by strip: a wave writes a strip of 16 rows
-    // x (16 NTO) columns (8 bytes per lane and column tile) into a window of its own and reads it
-    // back as 16 bytes per lane, LPR lanes to a row: every store instruction then writes whole row
-    // segments (128 bytes, a cache line, for four column tiles), where the accumulator layout by
-    // itself gives 32 bytes per row and instruction and the L2 writes some lines back more than
-    // once.  No barrier inside: a wave's LDS operations complete in order and the window is the
-    // wave's own (the stage ring is free: the K loop ended with every load landed and every wave
-    // past its last fragment read).
-    constexpr int SEG_B = NTO * 16 * 2;           // bytes of a strip's row
-    constexpr int SPITCH = SEG_B + 16;            // padded: rows 16 bytes apart modulo the bank span
-    constexpr int LPR = SEG_B / 16;               // lanes per row when reading back
-    constexpr int RPP = 64 / LPR;                 // rows per pass
-    constexpr bool kStaged = (64 % LPR == 0) && (RPP <= 16) && (16 % RPP == 0);
     if (kStaged && vec_ok && (d.ldc & 7) == 0 && (((uintptr_t)d.c & 15) == 0) && (d.c_bs[0] & 7) == 0 &&
         (d.c_bs[1] & 7) == 0 && m0 + BM <= d.store_m && out_n0 + out_bn <= d.store_n) {
         const lds_ptr win = lds + wave * (2 * 16 * SPITCH);
-        const int rrow = lane / LPR, rchunk = lane % LPR;
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const lds_ptr buf = win + (i & 1) * 16 * SPITCH;
@@ -601,7 +734,11 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
             for (int p = 0; p < 16 / RPP; ++p) {
                 const int r = p * RPP + rrow;
                 const u32x4 v = *(const lds_u32x4 *)(buf + r * SPITCH + rchunk * 16);
-                *(ARKMI_GLOBAL u32x4 *)(C + (int64_t)(m0 + wm * WTM + i * 16 + r) * d.ldc + col_w + rchunk * 8) = v;
+                const int row_g = m0 + wm * WTM + i * 16 + r;
+                *(ARKMI_GLOBAL u32x4 *)(C + (int64_t)row_g * d.ldc + col_w + rchunk * 8) = v;
+                if (fuse)
+                    *(ARKMI_GLOBAL u32x4 *)(fout + (int64_t)row_g * d.fuse_ld_out + col_w + rchunk * 8) =
+                        fused_store_values<T>(d.fuse_kind - 1, d.fuse_c_second != 0, v, oth[i][p]);
             }
         }
         s.sync();  // the windows lie in the stage ring, which the next task (or another op body) fills

@@ -48,10 +48,13 @@ const void *step_kernel_select(int families) {
     ARKMI_FAIL(ARKMI_UNSUPPORTED, "no one-op kernel holds the op families ", families, " of a fused task");
 }
 
-void step_kernel_launch(const void *kernel, const LoopProgram &prog, int group, int grid, int threads,
-                        int lds_bytes, hipStream_t stream) {
+void step_kernel_launch(const void *kernel, const LoopProgram &prog, LoopControl *ctl, HostMailbox *mb_dev,
+                        int group, int grid, int threads, int lds_bytes, uint64_t wait_ticks, hipStream_t stream) {
     LoopArgs a{};
     a.prog = prog;
+    // a body's bounded wait (the split of K) needs the abort word and the limit here too
+    a.ctl = ctl; a.mb = mb_dev;
+    a.wait_ticks = wait_ticks;
     // kernel boundaries order the ops: no dependency counters
     a.prog.waits = nullptr; a.prog.wait_spans = nullptr; a.prog.signal_map = nullptr; a.prog.dep_counters = nullptr;
     a.group = group;

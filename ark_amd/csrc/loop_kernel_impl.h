@@ -326,6 +326,7 @@ __device__ __forceinline__ void signal_rows(KArgs ka, const DevTaskGroup &g, int
 
 constexpr int kTasksDone = -2;     // returned by a body: the group has no more tasks for this workgroup
 constexpr int kTasksAborted = -3;  // a dependency wait gave up
+static_assert(kGemmAborted == kTasksAborted, "a matmul body reports an expired wait with the task loop's value");
 
 __device__ __forceinline__ KArgs uniform_kargs(KArgs p) {
     const uint64_t a = (uint64_t)(uintptr_t)p;
@@ -371,6 +372,7 @@ __device__ __forceinline__ int long_task_loop(KArgs ka, int gi, int t0, int tid,
                 !wait_for_rows(ka, g, task_index(g, id), tid, kLoopMaxThreads, epoch, control))
                 return kTasksAborted;
             follow = one(KARG(prog.ops) + g.op_begin, (int)id);
+            if (follow == kTasksAborted) return kTasksAborted;
         }
         const DevTaskGroup g = load_const(KARG(prog.groups) + gi);
         if (g.op_count > 1) return follow;  // the kernel runs the followers, signals, and calls again
@@ -387,8 +389,16 @@ ARKMI_BODY int gemm_body(KArgs ka_in, int gi, int t0, int tid, lds_ptr lds, unsi
     return long_task_loop(ka, __builtin_amdgcn_readfirstlane(gi), __builtin_amdgcn_readfirstlane(t0), tid,
                           __builtin_amdgcn_readfirstlane(epoch), s.lds - kLdsReserved, [&](const DevOp *op, int task) {
                               const GemmDesc g = load_const(&op->gemm);
-                              return gemm_tile<T, BM, BN, TRANS_B, EpilogueStore, TRANS_A, DUAL_B, SPLIT>(
-                                  g, task, s, EpilogueStore());
+                              if constexpr (SPLIT) {
+                                  auto poll = [&](unsigned int *word, unsigned int want) {
+                                      return poll_equals(word, want, BodyWait{&KARG(ctl)->abort, KARG(wait_ticks)});
+                                  };
+                                  return gemm_tile<T, BM, BN, TRANS_B, EpilogueStore, TRANS_A, DUAL_B, SPLIT>(
+                                      g, task, s, EpilogueStore(), poll);
+                              } else {
+                                  return gemm_tile<T, BM, BN, TRANS_B, EpilogueStore, TRANS_A, DUAL_B, SPLIT>(
+                                      g, task, s, EpilogueStore());
+                              }
                           });
 }
 

@@ -18,8 +18,8 @@ const void *loop_kernel_select(int families, int *chosen);
 // The one-task-group kernel of the smallest variant that covers `families`,
 // and its launch (one kernel per op, for the separate-kernel comparison).
 const void *step_kernel_select(int families);
-void step_kernel_launch(const void *kernel, const LoopProgram &prog, int group, int grid, int threads,
-                        int lds_bytes, hipStream_t stream);
+void step_kernel_launch(const void *kernel, const LoopProgram &prog, LoopControl *ctl, HostMailbox *mb_dev,
+                        int group, int grid, int threads, int lds_bytes, uint64_t wait_ticks, hipStream_t stream);
 void loop_kernel_prepare(const void *kernel, int lds_bytes);
 int loop_kernel_max_blocks_per_cu(const void *kernel, int threads, int lds_bytes);
 int loop_kernel_lds_reserved();

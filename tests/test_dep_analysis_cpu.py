@@ -50,13 +50,17 @@ def test_rows_feeding_matmuls_spans_by_first_principles():
     # producer 1 signals the block of its tile row; every block collects one signal per tile column
     assert mm1["SignalMap"] == [t // tiles_n for t in range(mm1["NumTasks"])]
     # consumer 2 waits for the tile rows of the first matmul that cover its own rows
+    # (4096 x 2048 x 4096 gives 256x256 tiles to half of the CUs: K is split, two tasks per tile)
     c2 = _cfg(plan, 2)
     bm2, bn2 = c2["TileShapeMNK"][:2]
     tiles_n2 = 2048 // bn2
+    tiles2 = mm2["NumTasks"] // c2.get("SplitK", 1)
+    assert c2.get("SplitK") == 2 and tiles2 == 128
     (w,) = mm2["Waits"]
     assert w["ProducerGroup"] == mm1["Group"] and w["Expect"] == tiles_n
     for t, (lo, hi) in enumerate(w["Spans"]):
-        r0, r1 = (t // tiles_n2) * bm2, (t // tiles_n2 + 1) * bm2
+        tile = t % tiles2
+        r0, r1 = (tile // tiles_n2) * bm2, (tile // tiles_n2 + 1) * bm2
         assert (lo, hi) == (r0 // bm, (r1 - 1) // bm), t
     assert "SignalMap" not in mm2  # nobody waits for the last group
     assert a["NumCounters"] == norm["NumTasks"] + 4096 // bm
@@ -134,10 +138,12 @@ def test_decoder_layer_replaces_every_barrier():
     # attention row block, and a tile row of bm_o rows spans bm_o / 128 of them
     (w,) = g["wo"]["Waits"]
     assert w["ProducerGroup"] == g["attn"]["Group"] and w["Expect"] == 32
-    bm_o = _cfg(plan, g["wo"]["Group"])["TileShapeMNK"][0]
-    tiles_n_o = 4096 // _cfg(plan, g["wo"]["Group"])["TileShapeMNK"][1]
+    c_o = _cfg(plan, g["wo"]["Group"])
+    bm_o = c_o["TileShapeMNK"][0]
+    tiles_n_o = 4096 // c_o["TileShapeMNK"][1]
+    tiles_o = g["wo"]["NumTasks"] // c_o.get("SplitK", 1)  # K split in two: both tasks of a tile wait alike
     for t, (lo, hi) in enumerate(w["Spans"]):
-        r0 = (t // tiles_n_o) * bm_o
+        r0 = ((t % tiles_o) // tiles_n_o) * bm_o
         assert (lo, hi) == (r0 // 128, (r0 + bm_o - 1) // 128), t
     # the down projection needs the SwiGLU rows of its tile and the residual it adds
     assert sorted(w["ProducerGroup"] for w in g["down"]["Waits"]) == sorted([g["wo"]["Group"], g["swiglu"]["Group"]])
@@ -286,3 +292,27 @@ def test_counted_barrier_with_a_local_hazard_keeps_the_plain_tile_order():
     off = plan_analysis(plan, 0)
     assert [s["Kind"] for s in off["Steps"]] == ["Tasks", "Tasks", "Barrier", "Tasks"]
     assert _tasks_steps(off)[1]["XcdRound"] == 256
+
+
+def test_split_matmuls_alternate_roles_and_move_the_split_point(monkeypatch):
+    """A matmul that splits K in two gives the sender the shorter part (its partial sums are on their
+    way while the finisher still multiplies), and consecutive split matmuls swap which half of the
+    tasks finishes, so that the same workgroups do not finish every time."""
+    m = Model()
+    blk = llama.TransformerBlock(m, 4096, 32, 11008, "bf16")
+    blk.forward(m.tensor([1, 2048, 4096], "bf16"), m.tensor([1, 2048, 1, 128], "bf16"),
+                m.tensor([1, 1, 2048, 2048], "bf16"), fused=True, causal=True)
+    plan = _plan(m)
+    names = ["norm1", "q", "k", "v", "attn", "wo", "norm2", "swiglu", "down"]
+
+    def split_steps():
+        g = dict(zip(names, _tasks_steps(plan_analysis(plan, 0))))
+        assert all("SplitAt" not in g[n] for n in ("norm1", "attn", "norm2", "swiglu"))
+        return [(g[n]["SplitAt"], g[n]["SplitFlip"]) for n in ("q", "k", "v", "wo", "down")]
+
+    assert split_steps() == [(2240, False), (2240, True), (2240, False), (2240, True), (5696, False)]
+    monkeypatch.setenv("ARKMI_SPLITK_ALTERNATE", "0")
+    monkeypatch.setenv("ARKMI_SPLITK_SKEW", "0")
+    assert split_steps() == [(2048, False)] * 4 + [(5504, False)]
+    monkeypatch.setenv("ARKMI_SPLITK_SKEW", "1000000")  # a part of K keeps at least four K tiles
+    assert split_steps() == [(4096 - 256, False)] * 4 + [(11008 - 256, False)]

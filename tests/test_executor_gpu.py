@@ -873,20 +873,26 @@ def test_cast_through_bytes(oracle, dtype):
 # ---------------------------------------------------------------- matmul with K split in two
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("trans_other", [False, True])
-def test_matmul_split_k(oracle, dtype, trans_other):
+@pytest.mark.parametrize("K,skew", [(8192, None), (4096, None), (4096, "0"), (1024, "100000")])
+def test_matmul_split_k(oracle, monkeypatch, dtype, trans_other, K, skew):
     """An output that gives 256x256 tiles to half of the CUs only (2048 x 4096, the decoder layer's
-    projections) is planned with SplitK 2: two tasks per tile, each multiplying half of K; the half
-    that finishes second adds the two.  Several iterations reuse the arrival counters; checked on
-    sampled rows against the oracle, and bit for bit against the same plan run one kernel per op."""
+    projections) is planned with SplitK 2 from K = 4096 on: two tasks per tile, one multiplying the
+    upper part of K and sending its partial sums, the other the lower part, adding the two and
+    finishing the tile.  Several iterations reuse the tiles' full/empty words; the split point is
+    moved (equal parts; the shortest sender's part a short K allows); checked on sampled rows
+    against the oracle, and bit for bit against the same plan run one kernel per op."""
     import torch
     from ark_amd import Model, Executor
-    M, N, K = 2048, 4096, 8192
+    M, N = 2048, 4096
+    if skew is not None:
+        monkeypatch.setenv("ARKMI_SPLITK_SKEW", skew)
     a = make(oracle, (M, K), dtype, 111, "uniform")
     b = make(oracle, (N, K) if trans_other else (K, N), dtype, 112, "normal", scale=0.05)
     m = Model()
     ta, tb = m.tensor(a.shape, dtype), m.tensor(b.shape, dtype)
     c = m.matmul(ta, tb, trans_other=trans_other)
-    plan = m.plan(device_id=0)
+    split = {"NumWarps": 8, "SramBytes": 131072, "TileShapeMNK": [256, 256, 64], "SplitK": 2, "NumTasks": 256}
+    plan = m.plan(device_id=0, config_rules=[lambda op, arch: json.dumps(split)] if K < 4096 else ())
     cfg = json.loads(plan)["TaskInfos"][0]["Ops"][0]["Config"]
     assert cfg["SplitK"] == 2 and cfg["TileShapeMNK"][:2] == [256, 256] and cfg["NumTasks"] == 2 * 8 * 16, cfg
     (got,), ex, _ = run_model(m, {ta: a, tb: b}, [c], iters=3, plan=plan)
@@ -903,8 +909,8 @@ def test_matmul_split_k(oracle, dtype, trans_other):
 
 
 def test_matmul_split_k_with_follower_and_neighbours(oracle):
-    """The residual add fused behind a split matmul runs on the workgroup that finishes the tile; the
-    ops before and after it keep their grid barriers (a split tile has no fixed workgroup)."""
+    """The residual add fused behind a split matmul belongs to the workgroup that finishes the tile; the
+    ops before and after it keep their grid barriers (a split tile's sender is another workgroup)."""
     from ark_amd import Model
     dtype = "bf16"
     M, N, K = 2048, 4096, 8192

@@ -349,8 +349,9 @@ def test_rocm950_matmul_tile_choice():
         c = json.loads(m.plan(arch="ROCM_950", num_processors=256))["TaskInfos"][0]["Ops"][0]["Config"]
         return c["TileShapeMNK"][:2], c["NumTasks"]
     assert tile(8192, 11008, 4096) == ([256, 256], 32 * 43)
-    assert tile(2048, 4096, 4096) == ([256, 128], 8 * 32)         # 256x256 would leave CUs idle
-    assert tile(4096, 2048, 4096) == ([256, 128], 16 * 16)        # (of the half-size tiles the 256-row one first)
+    assert tile(2048, 4096, 2048) == ([256, 128], 8 * 32)         # 256x256 would leave CUs idle
+    assert tile(4096, 2048, 2048) == ([256, 128], 16 * 16)        # (of the half-size tiles the 256-row one first)
+    assert tile(2048, 4096, 4096) == ([256, 256], 2 * 8 * 16)     # K of 4096 or more: large tiles, K split in two
     assert tile(128 * 33, 4096, 4096) == ([128, 256], 33 * 16)    # 33 tile rows of 128: no 256-row tile divides
     assert tile(2048, 4096, 11008 // 128 * 128) == ([256, 256], 2 * 8 * 16)  # long K: large tiles, K split in two
     assert tile(2048, 2048, 128, batch=(1, 32)) == ([256, 256], 32 * 64)
@@ -401,7 +402,9 @@ def test_rocm950_matmul_tiles_and_split_k():
     assert c["TileShapeMNK"][:2] == [256, 256] and c["SplitK"] == 2 and c["NumTasks"] == 256
     c = cfg(2048, 4096, 11008, trans_other=True)
     assert c["SplitK"] == 2 and c["NumTasks"] == 256
-    c = cfg(2048, 4096, 4096)                       # the exchange of partial sums would cost what the tile gains
+    c = cfg(2048, 4096, 4096)                       # from K = 4096 on the split beats smaller tiles
+    assert c["TileShapeMNK"][:2] == [256, 256] and c["SplitK"] == 2 and c["NumTasks"] == 256
+    c = cfg(2048, 4096, 2048)                       # below, the exchange of partial sums costs what the tile gains
     assert "SplitK" not in c and c["TileShapeMNK"][:2] == [256, 128] and c["NumTasks"] == 256
     c = cfg(2048, 2048, 4096)                       # 64 large tiles: smaller tiles fill the chip instead
     assert "SplitK" not in c and c["TileShapeMNK"][:2] == [128, 128]
