@@ -1331,7 +1331,6 @@ struct Executor {
         h_group_fam.clear();
         group_sched_step.clear();
         int max_slot_lds = 0;
-        int n_split_matmuls = 0;
         trace_len = 0;
         const Json &task_infos = plan.at("TaskInfos");
         // A barrier of the reference's schedule orders *processors*, whether
@@ -1464,19 +1463,6 @@ struct Executor {
                             ARK_ERR(UnsupportedError, "task ", st.task_info, ": only elementwise ops can be fused "
                                     "behind a matmul");
                     }
-                }
-                if (ops[(size_t)g.op_begin].kind == DEV_GEMM && ops[(size_t)g.op_begin].gemm.split_k == 2) {
-                    // Split matmuls alternate which half of their tasks sends and which finishes:
-                    // a finisher works ~10 us longer than its sender, and with the same
-                    // workgroups finishing every time (Q, K, V projections in a row, no barrier
-                    // between them) the others would idle for the sum.  Only where a workgroup
-                    // runs at most one task of the matmul (see GemmDesc::split_flip).
-                    const char *env = getenv("ARKMI_SPLITK_ALTERNATE");
-                    const int n_tasks = (st.task_e - st.task_b + st.task_s - 1) / st.task_s;
-                    const int n_procs = (st.proc_e - st.proc_b + st.proc_s - 1) / st.proc_s;
-                    if (env && atoi(env) == 1 && st.n_slots == 1 && n_tasks <= n_procs)
-                        ops[(size_t)g.op_begin].gemm.split_flip = n_split_matmuls & 1;
-                    ++n_split_matmuls;
                 }
                 group_fused.push_back(g.op_count == 2 && fold_into_store(ops[(size_t)g.op_begin],
                                                                           ops[(size_t)g.op_begin + 1]) ? 1 : 0);
@@ -2605,7 +2591,6 @@ int arkmi_plan_analysis(const char *plan_json, int dep_counters, char **analysis
                     j["XcdBand"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.xcd_band;
                     if (ex.dry_ops[(size_t)g.op_begin].gemm.split_k == 2) {
                         j["SplitAt"] = (long long)ex.dry_ops[(size_t)g.op_begin].gemm.split_at;
-                        j["SplitFlip"] = ex.dry_ops[(size_t)g.op_begin].gemm.split_flip != 0;
                     }
                 }
                 j["Claimed"] = g.claim >= 0;

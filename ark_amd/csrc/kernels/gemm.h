@@ -77,10 +77,7 @@ struct GemmDesc {
     int32_t fuse_ld_other;     // elements between rows of the other operand (0: one row for all)
     int32_t fuse_ld_out;       // elements between rows of the result
     int32_t fuse_period;       // > 0: the other operand's column is taken modulo this (a multiple of 8)
-    // split_k == 2: 1 swaps the roles, tasks [0, tiles) finish and tasks [tiles, 2 tiles) send (set
-    // only where a workgroup runs one task of the matmul: a finisher must never stand in front of
-    // a sender on the same workgroup)
-    int32_t split_flip;
+    int32_t pad2_;
 };
 
 // Eight values of C (as stored) and eight of the other operand through elementwise op `op`,
@@ -127,7 +124,7 @@ __device__ __forceinline__ bool poll_equals(unsigned int *word, unsigned int wan
     unsigned polls = 0;
     while (__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != want) {
         __builtin_amdgcn_s_sleep(1);
-        if ((++polls & 63u) == 0) {
+        if ((++polls & 63u) == 0 && w.abort != nullptr) {  // (no abort word: nothing bounds the wait)
             if (__hip_atomic_load(w.abort, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
             if (wall_clock64() - t0 > w.limit_ticks) {
                 __hip_atomic_store(w.abort, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -218,11 +215,11 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     static_assert(!SPLIT || (!DUAL_B && !TRANS_A), "the split of K exists for plain matmuls");
     // split: tasks [0, tiles) send the part of K from split_at on, tasks [tiles, 2 tiles) multiply
     // the part below it and finish the tile.  A workgroup runs its tasks in rising order, so a
-    // sender never stands behind a finisher that waits for it.  (split_flip swaps the two roles.)
+    // sender never stands behind a finisher that waits for it.
     int task = task_in, k_begin = 0, k_len = d.k, half = 0;
     if constexpr (SPLIT) {
         const int tiles = d.tiles_m * d.tiles_n * d.batch_total;
-        half = (task_in >= tiles ? 0 : 1) ^ (d.split_flip ? 1 : 0);
+        half = task_in >= tiles ? 0 : 1;
         task = task_in >= tiles ? task_in - tiles : task_in;
         k_begin = half ? d.split_at : 0;
         k_len = half ? d.k - d.split_at : d.split_at;

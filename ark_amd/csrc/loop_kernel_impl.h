@@ -840,7 +840,11 @@ __global__ __launch_bounds__(kLoopMaxThreads) void arkmi_step_kernel(LoopArgs) {
     const KArgs ka = kernel_kargs();
     init_lds_control();
     const LoopProgram P = KARG(prog);
-    run_group<FAM>(ka, P, KARG(group), 1u);
+    if (!run_group<FAM>(ka, P, KARG(group), 1u) && threadIdx.x == 0) {
+        // a body's bounded wait expired: report it the way the loop kernel does
+        HostMailbox *mb = KARG(mb);
+        if (mb) __hip_atomic_store(&mb->status, (int)MB_ABORTED, __ATOMIC_RELAXED, SYSTEM);
+    }
 }
 
 // Defines the host-visible handles of one kernel variant; each variant is its own

@@ -294,10 +294,9 @@ def test_counted_barrier_with_a_local_hazard_keeps_the_plain_tile_order():
     assert _tasks_steps(off)[1]["XcdRound"] == 256
 
 
-def test_split_matmuls_alternate_roles_and_move_the_split_point(monkeypatch):
-    """A matmul that splits K in two gives the sender the shorter part (its partial sums are on their
-    way while the finisher still multiplies), and consecutive split matmuls swap which half of the
-    tasks finishes, so that the same workgroups do not finish every time."""
+def test_split_matmuls_give_the_sender_the_shorter_part(monkeypatch):
+    """A matmul that splits K in two gives the sender the shorter part: its partial sums are on their
+    way while the finisher still multiplies.  The split point is reported by the analysis."""
     m = Model()
     blk = llama.TransformerBlock(m, 4096, 32, 11008, "bf16")
     blk.forward(m.tensor([1, 2048, 4096], "bf16"), m.tensor([1, 2048, 1, 128], "bf16"),
@@ -305,14 +304,13 @@ def test_split_matmuls_alternate_roles_and_move_the_split_point(monkeypatch):
     plan = _plan(m)
     names = ["norm1", "q", "k", "v", "attn", "wo", "norm2", "swiglu", "down"]
 
-    def split_steps():
+    def split_points():
         g = dict(zip(names, _tasks_steps(plan_analysis(plan, 0))))
         assert all("SplitAt" not in g[n] for n in ("norm1", "attn", "norm2", "swiglu"))
-        return [(g[n]["SplitAt"], g[n]["SplitFlip"]) for n in ("q", "k", "v", "wo", "down")]
+        return [g[n]["SplitAt"] for n in ("q", "k", "v", "wo", "down")]
 
-    assert split_steps() == [(2240, False), (2240, True), (2240, False), (2240, True), (5696, False)]
-    monkeypatch.setenv("ARKMI_SPLITK_ALTERNATE", "0")
+    assert split_points() == [2240] * 4 + [5696]
     monkeypatch.setenv("ARKMI_SPLITK_SKEW", "0")
-    assert split_steps() == [(2048, False)] * 4 + [(5504, False)]
+    assert split_points() == [2048] * 4 + [5504]
     monkeypatch.setenv("ARKMI_SPLITK_SKEW", "1000000")  # a part of K keeps at least four K tiles
-    assert split_steps() == [(4096 - 256, False)] * 4 + [(11008 - 256, False)]
+    assert split_points() == [4096 - 256] * 4 + [11008 - 256]

@@ -145,33 +145,3 @@ def test_residual_add_behind_a_split_matmul(oracle, monkeypatch):
     ref = oracle.binary(np.ascontiguousarray(r[pick]),
                         oracle.matmul(np.ascontiguousarray(x[pick]), w, dtype, trans_b=True), "add", dtype)
     _close_sum(oracle, ref, on[0][pick], dtype)
-
-
-def test_two_split_matmuls_in_a_row_swap_roles(oracle, monkeypatch):
-    """Two projections of one input with no barrier between them, both planned with K split in two:
-    the second swaps which half of its tasks sends and which finishes.  The same bits with the roles
-    fixed, and the oracle's values."""
-    from ark_amd import Model, plan_analysis
-    dtype = "bf16"
-    M, N, K = 2048, 4096, 4096
-    x = make(oracle, (M, K), dtype, 341, "normal")
-    w1 = make(oracle, (N, K), dtype, 342, "normal", scale=0.02)
-    w2 = make(oracle, (N, K), dtype, 343, "normal", scale=0.02)
-    res = []
-    for alt in ("1", "0"):
-        monkeypatch.setenv("ARKMI_SPLITK_ALTERNATE", alt)
-        m = Model()
-        tx, t1, t2 = m.tensor(x.shape, dtype), m.tensor(w1.shape, dtype), m.tensor(w2.shape, dtype)
-        y1 = m.matmul(tx, t1, trans_other=True)
-        y2 = m.matmul(tx, t2, trans_other=True)
-        plan = m.plan(device_id=0)
-        steps = [s for s in plan_analysis(plan)["Steps"] if s["Kind"] == "Tasks"]
-        assert [s["SplitFlip"] for s in steps] == ([False, True] if alt == "1" else [False, False])
-        got, _, _ = run_model(m, {tx: x, t1: w1, t2: w2}, [y1, y2], iters=3, plan=plan)
-        res.append(got)
-    assert np.array_equal(res[0][0], res[1][0]) and np.array_equal(res[0][1], res[1][1])
-    pick = np.sort(np.random.default_rng(8).choice(M, 32, replace=False))
-    pick[0], pick[-1] = 0, M - 1
-    xp = np.ascontiguousarray(x[pick])
-    close(oracle, oracle.matmul(xp, w1, dtype, trans_b=True), res[0][0][pick], dtype, 1e-2)
-    close(oracle, oracle.matmul(xp, w2, dtype, trans_b=True), res[0][1][pick], dtype, 1e-2)
