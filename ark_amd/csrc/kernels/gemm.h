@@ -586,15 +586,18 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     constexpr int LPR = SEG_B / 16;               // lanes per row when reading back
     constexpr int RPP = 64 / LPR;                 // rows per pass
     constexpr bool kStaged = (64 % LPR == 0) && (RPP <= 16) && (16 % RPP == 0);
-    // An elementwise op folded into the store (fuse_kind): the other operand's segments of the whole
-    // tile are requested ahead of the strips, which take a fraction of a memory round trip each
-    // (fetched one strip ahead, every strip waited for its segment): all of them here; for a
-    // split tile the first quarter here, before the finisher waits for and adds the sender's
-    // partial sums, and the rest after (the registers do not hold both at once).
+    // An elementwise op folded into the store (fuse_kind): the other operand's segments are
+    // requested four strips ahead of their use (a strip takes a fraction of a memory round trip:
+    // fetched one strip ahead, every strip waited for its segment).  The first four strips' here;
+    // for a split tile two of them here, before the finisher waits for and adds the sender's
+    // partial sums, and two after (the registers do not hold more beside the sums being added).
     constexpr int PASSES = kStaged ? 16 / RPP : 1;
     const int rrow = lane / LPR, rchunk = lane % LPR;
     const bool fuse = !DUAL_B && kStaged && d.fuse_kind != 0 && (!SPLIT || half == 0);
-    u32x4 oth[MT][PASSES];
+    // (four strips: with all eight of a 256-row tile requested at once, 64 more registers, the
+    // kernel spilled 17 registers to scratch in every variant, and a plain 4096^3 matmul lost 4 %)
+    constexpr int FW = MT < 4 ? MT : 4;  // strips requested ahead
+    u32x4 oth[FW][PASSES];
     gptr<const T> other = as_global(static_cast<const T *>(d.fuse_other));
     gptr<T> fout = as_global(static_cast<T *>(d.fuse_out));
     int ocol = col_w + rchunk * 8;
@@ -606,7 +609,7 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
             dst[p] = *(const ARKMI_GLOBAL u32x4 *)(other + (int64_t)row * d.fuse_ld_other + ocol);
         }
     };
-    constexpr int FIRST = SPLIT ? (MT + 3) / 4 : MT;
+    constexpr int FIRST = SPLIT ? (FW < 2 ? FW : 2) : FW;
     if (fuse) {
 #pragma unroll
         for (int i = 0; i < FIRST; ++i) other_load(i, oth[i]);
@@ -648,10 +651,7 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
             return -1;
         }
         // the finisher: AHEAD row tiles of loads in flight while one is added
-#ifndef ARKMI_SPLIT_AHEAD
-#define ARKMI_SPLIT_AHEAD 4
-#endif
-        constexpr int AHEAD = MT < ARKMI_SPLIT_AHEAD ? MT : ARKMI_SPLIT_AHEAD;
+        constexpr int AHEAD = MT < 4 ? MT : 4;
         u32x4 in[AHEAD][NT];
 #pragma unroll
         for (int i = 0; i < AHEAD; ++i)
@@ -678,7 +678,7 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
 
     if (fuse) {
 #pragma unroll
-        for (int i = FIRST; i < MT; ++i) other_load(i, oth[i]);
+        for (int i = FIRST; i < FW; ++i) other_load(i, oth[i]);
     }
 
     // ---- epilogue: lane (m = lane%16, g = lane/16) holds C[m][4g .. 4g+3] of each 16x16 tile ----
@@ -714,30 +714,40 @@ __device__ __forceinline__ int gemm_tile(const GemmDesc &d, int task_in, const S
     if (kStaged && vec_ok && (d.ldc & 7) == 0 && (((uintptr_t)d.c & 15) == 0) && (d.c_bs[0] & 7) == 0 &&
         (d.c_bs[1] & 7) == 0 && m0 + BM <= d.store_m && out_n0 + out_bn <= d.store_n) {
         const lds_ptr win = lds + wave * (2 * 16 * SPITCH);
+        // (two copies of the strip loop, chosen per tile: with the folded op's branches inside the
+        // one loop its stores no longer ran together, and a matmul with nothing folded lost 2 %)
+        auto strips = [&](auto folded_c) {
+            constexpr bool FOLDED = decltype(folded_c)::value;
 #pragma unroll
-        for (int i = 0; i < MT; ++i) {
-            const lds_ptr buf = win + (i & 1) * 16 * SPITCH;
-            const int row = m0 + wm * WTM + i * 16 + l16;
+            for (int i = 0; i < MT; ++i) {
+                const lds_ptr buf = win + (i & 1) * 16 * SPITCH;
+                const int row = m0 + wm * WTM + i * 16 + l16;
 #pragma unroll
-            for (int j = 0; j < NTO; ++j) {
-                float o[4];
-                value4(i, j, row, col_w + j * 16 + 4 * g4, o);
-                T t[4] = {from_f32<T>(o[0]), from_f32<T>(o[1]), from_f32<T>(o[2]), from_f32<T>(o[3])};
-                u32x2 w;
-                __builtin_memcpy(&w, t, 8);
-                *(__attribute__((address_space(3))) u32x2 *)(buf + l16 * SPITCH + j * 32 + g4 * 8) = w;
+                for (int j = 0; j < NTO; ++j) {
+                    float o[4];
+                    value4(i, j, row, col_w + j * 16 + 4 * g4, o);
+                    T t[4] = {from_f32<T>(o[0]), from_f32<T>(o[1]), from_f32<T>(o[2]), from_f32<T>(o[3])};
+                    u32x2 w;
+                    __builtin_memcpy(&w, t, 8);
+                    *(__attribute__((address_space(3))) u32x2 *)(buf + l16 * SPITCH + j * 32 + g4 * 8) = w;
+                }
+#pragma unroll
+                for (int p = 0; p < 16 / RPP; ++p) {
+                    const int r = p * RPP + rrow;
+                    const u32x4 v = *(const lds_u32x4 *)(buf + r * SPITCH + rchunk * 16);
+                    const int row_g = m0 + wm * WTM + i * 16 + r;
+                    *(ARKMI_GLOBAL u32x4 *)(C + (int64_t)row_g * d.ldc + col_w + rchunk * 8) = v;
+                    if constexpr (FOLDED)
+                        *(ARKMI_GLOBAL u32x4 *)(fout + (int64_t)row_g * d.fuse_ld_out + col_w + rchunk * 8) =
+                            fused_store_values<T>(d.fuse_kind - 1, d.fuse_c_second != 0, v, oth[i % FW][p]);
+                }
+                if constexpr (FOLDED) {
+                    if (i + FW < MT) other_load(i + FW, oth[i % FW]);
+                }
             }
-#pragma unroll
-            for (int p = 0; p < 16 / RPP; ++p) {
-                const int r = p * RPP + rrow;
-                const u32x4 v = *(const lds_u32x4 *)(buf + r * SPITCH + rchunk * 16);
-                const int row_g = m0 + wm * WTM + i * 16 + r;
-                *(ARKMI_GLOBAL u32x4 *)(C + (int64_t)row_g * d.ldc + col_w + rchunk * 8) = v;
-                if (fuse)
-                    *(ARKMI_GLOBAL u32x4 *)(fout + (int64_t)row_g * d.fuse_ld_out + col_w + rchunk * 8) =
-                        fused_store_values<T>(d.fuse_kind - 1, d.fuse_c_second != 0, v, oth[i][p]);
-            }
-        }
+        };
+        if (fuse) strips(std::true_type{});
+        else strips(std::false_type{});
         s.sync();  // the windows lie in the stage ring, which the next task (or another op body) fills
         return task;
     }

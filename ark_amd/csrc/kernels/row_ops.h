@@ -52,7 +52,13 @@ struct RowOpDesc {
     // 1: a later op of the plan reads the input again (before anything overwrites it): fetch it
     // through the caches instead of streaming past them
     int32_t in_read_again;
-    int32_t pad_;
+    // The row op that runs next on the same workgroups with the same dealing of rows (the host knows;
+    // pf_base null: none): while a wave finishes its last row of this task it touches the lines of
+    // its first row of that op, pf_base + first row * pf_row_bytes, pf_len bytes, so that the next
+    // task's first loads, which nothing overlaps, find them in the L2.
+    int32_t pf_len;
+    const void *pf_base;
+    int64_t pf_row_bytes;
 };
 
 __device__ __forceinline__ int64_t row_offset(int64_t r, int dim_c, int dim_h,
@@ -433,24 +439,36 @@ __device__ __forceinline__ void row_op_pipelined(const RowOpDesc &d, int64_t row
         s.sync();
         w_lds = s.lds;
     }
-    for (int j = 0; j < count; ++j) {
-        const int64_t row = row0 + (int64_t)j * stride;
-        const bool more = j + 1 < count;
-        if (more)
-            row_exact_load<T, NC>(
-                as_global(static_cast<const T *>(d.in) + row_offset(row + stride, d.dim_c, d.dim_h, d.in_s)), lane,
-                nxt, d.in_read_again != 0);
-        __builtin_amdgcn_sched_barrier(0);
+    uint32_t touched = 0;
+    auto finish = [&](int64_t row) {
         gptr<T> out = as_global(static_cast<T *>(d.out) + row_offset(row, d.dim_c, d.dim_h, d.out_s));
         gptr<const T> mask = nullptr;
         if (KIND == ROW_SOFTMAX && d.weight)
             mask = as_global(static_cast<const T *>(d.weight) + row_offset(row, d.dim_c, d.dim_h, d.w_s));
         row_exact_finish<T, KIND, NC>(d, cur, out, lane, mask, w_lds, cur, false);
-        if (more) {
+    };
+    // every row but the last: the next row's loads are issued, then this one is reduced and stored
+    for (int j = 0; j + 1 < count; ++j) {
+        const int64_t row = row0 + (int64_t)j * stride;
+        row_exact_load<T, NC>(
+            as_global(static_cast<const T *>(d.in) + row_offset(row + stride, d.dim_c, d.dim_h, d.in_s)), lane, nxt,
+            d.in_read_again != 0);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(row);
 #pragma unroll
-            for (int c = 0; c < NC; ++c) cur[c] = nxt[c];
-        }
+        for (int c = 0; c < NC; ++c) cur[c] = nxt[c];
     }
+    // the last row (kept out of the loop above, which then has no branch inside): in place of a next
+    // row's loads, one word of every 128-byte line of the next op's first row for this wave
+    if (count > 0) {
+        if (d.pf_base) {
+            const ARKMI_GLOBAL char *p = (const ARKMI_GLOBAL char *)d.pf_base + row0 * d.pf_row_bytes;
+            for (int b = lane * 128; b < d.pf_len; b += kWave * 128) touched ^= *(const ARKMI_GLOBAL uint32_t *)(p + b);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        finish(row0 + (int64_t)(count - 1) * stride);
+    }
+    asm volatile("" ::"v"(touched));  // (the touches are waited for here, behind the last row's stores)
 }
 
 // RMSNorm with one row per wave and task: the weights (the same NC vectors per lane for every

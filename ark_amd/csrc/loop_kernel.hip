@@ -22,6 +22,7 @@ const void *loop_kernel_variant_32();  // the rarely used bodies alone
 const void *loop_kernel_variant_63();  // everything but the split of K
 const void *loop_kernel_variant_68();  // GEMM incl. the split of K
 const void *loop_kernel_variant_70();  // elementwise + GEMM incl. the split of K
+const void *loop_kernel_variant_85();  // rows + GEMM incl. the split of K + attention (elementwise ops all folded)
 const void *loop_kernel_variant_87();  // rows + elementwise + GEMM incl. the split of K + attention
 const void *loop_kernel_variant_127(); // everything
 
@@ -71,7 +72,8 @@ const void *loop_kernel_select(int families, int *chosen) {
         {3, loop_kernel_variant_3},   {11, loop_kernel_variant_11}, {4, loop_kernel_variant_4},
         {6, loop_kernel_variant_6},   {7, loop_kernel_variant_7},   {23, loop_kernel_variant_23},
         {31, loop_kernel_variant_31}, {63, loop_kernel_variant_63},
-        {68, loop_kernel_variant_68}, {70, loop_kernel_variant_70}, {87, loop_kernel_variant_87},
+        {68, loop_kernel_variant_68}, {70, loop_kernel_variant_70}, {85, loop_kernel_variant_85},
+        {87, loop_kernel_variant_87},
         {127, loop_kernel_variant_127},
     };
     for (const Variant &v : table) {

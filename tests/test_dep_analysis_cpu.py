@@ -112,7 +112,9 @@ def test_decoder_layer_replaces_every_barrier():
     off, on = plan_analysis(plan, 0), plan_analysis(plan, 1)
     assert off["BarriersCounted"] == 0 and [s["Kind"] for s in off["Steps"]].count("Barrier") == 6
     assert on["BarriersCounted"] == 6 and "Barrier" not in [s["Kind"] for s in on["Steps"]]
-    assert on["KernelFamilies"] == off["KernelFamilies"] == 87
+    # rows + matmul + split of K + attention: the rotation and the residual adds are folded into the
+    # projections' stores and need no elementwise body in the kernel
+    assert on["KernelFamilies"] == off["KernelFamilies"] == 85
     groups = _tasks_steps(on)
     names = ["norm1", "q", "k", "v", "attn", "wo", "norm2", "swiglu", "down"]
     g = dict(zip(names, groups))
@@ -314,3 +316,51 @@ def test_split_matmuls_give_the_sender_the_shorter_part(monkeypatch):
     assert split_points() == [2048] * 4 + [5504]
     monkeypatch.setenv("ARKMI_SPLITK_SKEW", "1000000")  # a part of K keeps at least four K tiles
     assert split_points() == [4096 - 256] * 4 + [11008 - 256]
+
+
+def test_row_ops_touch_the_first_rows_of_the_row_op_that_follows(monkeypatch):
+    """Row ops that follow one another on the same workgroups with the same dealing of rows, and no grid
+    barrier between them, are linked: each touches its waves' first rows of the next while it finishes
+    (a hint that costs a load per wave).  A matmul in between, another row count or a kept barrier
+    breaks the link."""
+    def flags(m):
+        a = plan_analysis(_plan(m), 0)
+        return [s.get("TouchesNextRows") for s in _tasks_steps(a)], a["IterationSync"]
+
+    m = Model()
+    x, w = m.tensor([16384, 4096], "fp16"), m.tensor([1, 4096], "fp32")
+    m.reduce_sum(x, axis=1)
+    m.softmax(x)
+    m.rmsnorm(x, w, 1e-5)
+    got, it_sync = flags(m)
+    # reduce_sum and softmax leave X in the caches for the op behind them (InputReadAgain): nothing to
+    # touch there, and nothing ahead of a reader that fetches through the caches (the first op of the
+    # next iteration)
+    assert got == [False, False, False]
+    monkeypatch.setenv("ARKMI_ROW_CACHED_INPUT", "0")   # every op streams: each touches the next one's rows
+    assert flags(m)[0] == [True, True, it_sync != 2]
+    monkeypatch.delenv("ARKMI_ROW_CACHED_INPUT")
+    m2 = Model()
+    xs = [m2.tensor([16384, 4096], "fp16") for _ in range(3)]
+    for x in xs:
+        m2.softmax(x)
+    got2, it_sync2 = flags(m2)
+    assert got2 == [True, True, it_sync2 != 2]  # different inputs, streamed: each touches the next one's rows
+    monkeypatch.setenv("ARKMI_ROW_PREFETCH", "0")
+    assert flags(m)[0] == [False, False, False]
+    monkeypatch.delenv("ARKMI_ROW_PREFETCH")
+
+    m = Model()
+    x, y = m.tensor([16384, 4096], "fp16"), m.tensor([8192, 4096], "fp16")
+    m.softmax(x)
+    m.softmax(y)            # half the rows: another dealing
+    m.matmul(m.tensor([4096, 4096], "fp16"), m.tensor([4096, 4096], "fp16"))
+    got, _ = flags(m)
+    assert got[0] is False and got[1] is False and got[2] is None
+
+    m = Model()
+    x = m.tensor([16384, 4096], "fp16")
+    m.softmax(m.softmax(x))  # linked exactly when no grid barrier stays between the two
+    a = plan_analysis(_plan(m), 0)
+    kinds = [s["Kind"] for s in a["Steps"]]
+    assert _tasks_steps(a)[0]["TouchesNextRows"] == ("Barrier" not in kinds[:kinds.index("Tasks", 1)])
