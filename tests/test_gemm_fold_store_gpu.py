@@ -145,3 +145,33 @@ def test_residual_add_behind_a_split_matmul(oracle, monkeypatch):
     ref = oracle.binary(np.ascontiguousarray(r[pick]),
                         oracle.matmul(np.ascontiguousarray(x[pick]), w, dtype, trans_b=True), "add", dtype)
     _close_sum(oracle, ref, on[0][pick], dtype)
+
+
+@pytest.mark.parametrize("onto", ["other", "c"])
+def test_result_written_over_an_operand(oracle, monkeypatch, onto):
+    """The op's output may be one of its inputs: the residual it adds (h <- h + x @ w, the way a decoder
+    layer updates its hidden state in place) or the matmul's own result.  A lane loads its segment of the
+    other operand before it stores the same addresses, and stores C before the result."""
+    dtype = "bf16"
+    M, N, K = 512, 512, 256
+    x = make(oracle, (M, K), dtype, 351)
+    w = make(oracle, (N, K), dtype, 352, "normal", scale=0.05)
+    r = make(oracle, (M, N), dtype, 353)
+
+    def build(m):
+        tx, tw, tr = m.tensor(x.shape, dtype), m.tensor(w.shape, dtype), m.tensor(r.shape, dtype)
+        with m.planner_context(sync=False):
+            y = m.matmul(tx, tw, trans_other=True)
+            o = m.add(tr, y, tr if onto == "other" else y)
+        return (tx, tw, tr), [o]
+
+    (plan, on_flags, on), (_, off_flags, off) = _both_ways(
+        monkeypatch, build, lambda t: {t[0]: x, t[1]: w, t[2]: r})
+    assert len(json.loads(plan)["TaskInfos"]) == 1 and on_flags == [True] and off_flags == [False]
+    assert np.array_equal(on[0], off[0])
+    # (two iterations: written over the residual, the second adds the product to the first's result)
+    y = oracle.matmul(x, w, dtype, trans_b=True)
+    ref = oracle.binary(r, y, "add", dtype)
+    if onto == "other":
+        ref = oracle.binary(ref, y, "add", dtype)
+    _close_sum(oracle, ref, on[0], dtype)
