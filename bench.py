@@ -12,7 +12,9 @@ third read may be served by that cache (the plan keeps X cacheable for them on p
 of algorithmic bytes).
 
 `value` is the whole-job throughput of the timed run of the resident loop kernel (host clock
-around run() + wait(), inputs already in HBM) in algorithmic GB/s.  `roofline` prices the
+around run() + wait(), inputs already in HBM) in algorithmic GB/s: the kernel is loaded for 30 ms
+untimed first (the chip leaves its idle clocks over tens of milliseconds), then come the W
+warm-up steps and exactly K timed ones.  `roofline` prices the
 loop kernel itself against 8 TB/s: the same plan launched in one-shot mode (the kernel runs
 its iterations and returns) under HIP events on the stream it is launched on, which is the
 dispatch `rocprofv3 --kernel-trace` reports.  `roofline.frac` counts algorithmic bytes and so
@@ -605,6 +607,15 @@ def main():
     # The loop kernel stays resident between run() calls, so a device-wide synchronize inside
     # the timed region would wait for it to leave; Executor.wait() is the completion point.
     ex.launch()
+    # Untimed load on this kernel as well, 30 ms of it in batches of the timed size: between the
+    # probes and the first command the chip has idled through the kernel's launch, and the `value`
+    # leg is meant to read the rate the resident kernel sustains, not the first milliseconds of a
+    # clock ramp (the same is done for every other resident figure of this file).  Then the W
+    # warm-up steps of the contract, then exactly K timed steps.
+    t_ramp = time.perf_counter()
+    while time.perf_counter() - t_ramp < 0.03:
+        ex.run(steps)
+        ex.wait()
     if warm:
         ex.run(warm)
         ex.wait()
