@@ -471,11 +471,11 @@ __device__ __forceinline__ void row_op_pipelined(const RowOpDesc &d, int64_t row
     asm volatile("" ::"v"(touched));  // (the touches are waited for here, behind the last row's stores)
 }
 
-// RMSNorm with one row per wave and task: the weights (the same NC vectors per lane for every
-// row) go straight to registers, fetched beside the row, instead of one dependent load per
-// chunk after the reduction, or a copy through LDS that a single row cannot repay (2048 rows of
-// 4096 bf16 in the loop kernel: 13.0 us with fp32 weights staged in LDS, 11.6 loaded chunk by
-// chunk, 8.3 with the weights in registers).
+// RMSNorm of 16-bit rows: the weights (the same NC vectors per lane for every row) go straight to
+// registers, fetched beside the first row, instead of one dependent load per chunk after the
+// reduction or a copy through LDS with two workgroup barriers per task (2048 rows of 4096 bf16,
+// one row per wave, in the loop kernel: 13.0 us with fp32 weights staged in LDS, 11.6 loaded
+// chunk by chunk, 8.3 with the weights in registers).
 template <typename T, int NC, bool W32>
 __device__ __forceinline__ void rmsnorm_rows_weight_in_regs(const RowOpDesc &d, int64_t row0, int stride, int count,
                                                             int lane) {
@@ -497,16 +497,37 @@ __device__ __forceinline__ void rmsnorm_rows_weight_in_regs(const RowOpDesc &d, 
 #pragma unroll
         for (int c = 0; c < NC; ++c) wreg[c] = load16<T>(wp + c * (kWave * VN) + lane * VN);
     }
-    for (int j = 0; j < count; ++j) {
-        const int64_t row = row0 + (int64_t)j * stride;
-        Vec16<T> reg[NC];
-        row_exact_load<T, NC>(as_global(static_cast<const T *>(d.in) + row_offset(row, d.dim_c, d.dim_h, d.in_s)),
-                              lane, reg, d.in_read_again != 0);
-        __builtin_amdgcn_sched_barrier(0);
+    // the rows as in row_op_pipelined: the next row's loads ahead of this row's reduction, the
+    // last row outside the loop, with the touches of the next op's first row in its place
+    Vec16<T> cur[NC], nxt[NC];
+    if (count > 0)
+        row_exact_load<T, NC>(as_global(static_cast<const T *>(d.in) + row_offset(row0, d.dim_c, d.dim_h, d.in_s)),
+                              lane, cur, d.in_read_again != 0);
+    uint32_t touched = 0;
+    auto finish = [&](int64_t row) {
         row_exact_finish<T, ROW_RMSNORM, NC>(
-            d, reg, as_global(static_cast<T *>(d.out) + row_offset(row, d.dim_c, d.dim_h, d.out_s)), lane, nullptr,
+            d, cur, as_global(static_cast<T *>(d.out) + row_offset(row, d.dim_c, d.dim_h, d.out_s)), lane, nullptr,
             nullptr, wreg, true);
+    };
+    for (int j = 0; j + 1 < count; ++j) {
+        const int64_t row = row0 + (int64_t)j * stride;
+        row_exact_load<T, NC>(
+            as_global(static_cast<const T *>(d.in) + row_offset(row + stride, d.dim_c, d.dim_h, d.in_s)), lane, nxt,
+            d.in_read_again != 0);
+        __builtin_amdgcn_sched_barrier(0);
+        finish(row);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) cur[c] = nxt[c];
     }
+    if (count > 0) {
+        if (d.pf_base) {
+            const ARKMI_GLOBAL char *p = (const ARKMI_GLOBAL char *)d.pf_base + row0 * d.pf_row_bytes;
+            for (int b = lane * 128; b < d.pf_len; b += kWave * 128) touched ^= *(const ARKMI_GLOBAL uint32_t *)(p + b);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        finish(row0 + (int64_t)(count - 1) * stride);
+    }
+    asm volatile("" ::"v"(touched));
 }
 
 // One task = rows_per_wave rows per wave of the slot.  With R rows per wave and W
@@ -532,7 +553,7 @@ __device__ __forceinline__ void row_op_task(const RowOpDesc &d, int task, const 
     const bool stage = (KIND == ROW_RMSNORM) && d.weight_lds != 0;
     if constexpr (KIND == ROW_RMSNORM && sizeof(T) == 2) {
         // (decided by the descriptor alone: the whole slot takes this path, which has no barrier)
-        if (ok && d.weight && R == 1) {
+        if (ok && d.weight) {
             if (d.weight_fp32) {
                 if (d.cols == 4 * PER_CHUNK) return rmsnorm_rows_weight_in_regs<T, 4, true>(d, row0, nw, count, s.lane());
                 if (d.cols == 8 * PER_CHUNK) return rmsnorm_rows_weight_in_regs<T, 8, true>(d, row0, nw, count, s.lane());
